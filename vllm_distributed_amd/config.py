@@ -139,6 +139,20 @@ def normalize_hf_config(cfg: Dict[str, Any]) -> None:
                      ("head_dim", first.get("dim")), ("tie_word_embeddings", False)):
             if cfg.get(k) is None and v is not None:
                 cfg[k] = v
+    if cfg.get("architecture") == "Gosizen" or cfg.get("model_type") == "gosizen":
+        # Gosizen lists its layers one by one too (a parallel mixer nests its two halves); no position table
+        cfg.setdefault("model_type", "gosizen")
+        cfg.setdefault("architectures", ["GosizenForCausalLM"])
+        mixers = [l.get("mixer") or {} for l in cfg.get("layers") or []]
+        first = mixers[0] if mixers else {}
+        first = first.get("left") or first
+        for k, v in (("hidden_size", cfg.get("width")), ("vocab_size", cfg.get("vocab")),
+                     ("max_position_embeddings", cfg.get("max_positions") or 131072), ("num_hidden_layers", len(mixers)),
+                     ("num_attention_heads", first.get("heads", 1)),
+                     ("num_key_value_heads", first.get("kv_heads") or first.get("heads", 1)),
+                     ("head_dim", first.get("dim")), ("tie_word_embeddings", False)):
+            if cfg.get(k) is None and v is not None:
+                cfg[k] = v
     if cfg.get("model_type") == "dbrx":
         # DBRX nests its attention and expert settings
         a, f = cfg.get("attn_config") or {}, cfg.get("ffn_config") or {}

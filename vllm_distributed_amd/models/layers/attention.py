@@ -224,12 +224,22 @@ def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None):
     ``{factor, original, fast, slow}`` blends towards ``f_i / factor`` the YaRN way: with ``d(r) = dims *
     ln(original / (2 pi r)) / (2 ln base)`` the index at which a pair turns ``r`` times within ``original``
     positions, a ramp rises linearly from 0 at ``max(floor(d(fast)), 0)`` to 1 at ``min(ceil(d(slow)), dims - 1)``;
-    pair ``i`` gets ``ramp_i f_i / factor + (1 - ramp_i) f_i``, and the factor is ``0.1 ln(factor) + 1``."""
+    pair ``i`` gets ``ramp_i f_i / factor + (1 - ramp_i) f_i``, and the factor is ``0.1 ln(factor) + 1``.
+    ``scaling`` = ``{factor, original, low, high}`` slows by wavelength bands instead (Llama 3.1's rule): with
+    ``l = 2 pi / f``, ``f`` stays where ``l < original / high``, becomes ``f / factor`` where ``l > original / low``,
+    and between the two is ``(1 - s) f / factor + s f`` with ``s = (original / l - low) / (high - low)``; factor 1."""
     import math
     i = torch.arange(dims // 2, dtype=torch.float64)
     f = float(base) ** (-2.0 * i / dims)
     scale = 1.0
-    if scaling:
+    if scaling and "low" in scaling and "high" in scaling:
+        factor, original = float(scaling["factor"]), float(scaling["original"])
+        low, high = float(scaling["low"]), float(scaling["high"])
+        wavelength = 2.0 * math.pi / f
+        s = (original / wavelength - low) / (high - low)
+        blended = (1.0 - s) * f / factor + s * f
+        f = torch.where(wavelength < original / high, f, torch.where(wavelength > original / low, f / factor, blended))
+    elif scaling:
         factor, original = float(scaling["factor"]), float(scaling["original"])
 
         def index_of(turns: float) -> float:
@@ -248,19 +258,28 @@ class RowLatentAttention(Attention):
     query and the output by the caller.  Any ``rank`` / ``rope``; the rotation is computed from ``inv_freq`` in the
     kernel (positions and angles in fp32), so no table bounds the positions; scores, softmax and the weighted sum are
     fp32 in every dtype.  ``source``: another layer's instance whose rows this layer reads instead of keeping its own
-    (layers that share keys and values: the reader allocates nothing and writes nothing)."""
+    (layers that share keys and values: the reader allocates nothing and writes nothing).  ``window``: a query sees
+    itself and the ``window - 1`` tokens before it (0: everything); ``sink``: a learned number per head whose
+    exponential joins the softmax denominator (a parameter, or another instance's parameter to share);
+    ``interleaved``: the rotation pairs neighbouring values instead of values half the rotated width apart."""
     latent = True
     row_cache = True
 
     def __init__(self, num_heads: int, rank: int, rope: int, scale: float, layer_idx: int,
-                 source: Optional["RowLatentAttention"] = None, dtype: Optional[torch.dtype] = None):
-        super().__init__(num_heads, rank + rope, 1, scale, layer_idx)
+                 source: Optional["RowLatentAttention"] = None, dtype: Optional[torch.dtype] = None,
+                 window: int = 0, sink=False, interleaved: bool = False):
+        super().__init__(num_heads, rank + rope, 1, scale, layer_idx, sliding_window=window)
         self.rank, self.rope, self.v_dim = rank, rope, rank
+        self.interleaved = bool(interleaved)
+        if isinstance(sink, nn.Parameter):
+            self.sink = sink
+        else:
+            self.sink = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32), requires_grad=False) if sink else None
         # where the matrix-core latent kernel is built for this width and type, the values are cached once more as
         # its V^T fragments and it serves the layer (with fp32-precise softmax weights); else the plain kernel
         on_gpu = torch.empty(0).device.type != "cpu"       # (modules are built under the target device)
-        self.fragments = bool(on_gpu and dtype is not None and rank % 16 == 0
-                              and ops.mla_kernel_ok(rank + rope, rank, dtype))
+        self.fragments = bool(on_gpu and dtype is not None and rank % 16 == 0 and not self.window
+                              and self.sink is None and ops.mla_kernel_ok(rank + rope, rank, dtype))
         if source is not None:
             self.fragments = source.fragments
         if source is not None and (source.rank, source.rope) != (rank, rope):
@@ -289,14 +308,15 @@ class RowLatentAttention(Attention):
 
     def forward_latent(self, q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
                        norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor,
-                       rot_scale: float) -> torch.Tensor:
+                       rot_scale: float, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``q[T, H, nope + rope]``, ``q_lat[H, T, rank]``, ``latent[T, rank + rope]`` (None for a reader of another
-        layer's rows): norm, rotations, cache write and query assembly in one op, then attention -> ``[T, H, rank]``."""
+        layer's rows): norm, rotations, cache write and query assembly in one op, then attention -> ``[T, H, rank]``;
+        ``gate[T, H]`` (raw): head ``h``'s result times ``sigmoid(gate[t, h])``."""
         md, pos = _CTX.attn_metadata, _CTX.positions
         write = latent is not None and self.source is None and md is not None
         qf = ops.latent_prep(q, nope, q_lat, latent if write else None, norm_weight, eps, inv_freq, rot_scale, pos,
                              self.k_cache if write else None, md.slot_mapping if write else None,
-                             self.v_cache if write and self.fragments else None)
+                             self.v_cache if write and self.fragments else None, self.interleaved)
         if md is None:                          # memory-profiling pass: no cache bound
             return qf[..., :self.rank].contiguous()
         rows, lens = md.token_rows(pos)
@@ -304,7 +324,8 @@ class RowLatentAttention(Attention):
             owner = self.source if self.source is not None else self
             return ops.mla_attention(qf, owner.k_cache, owner.v_cache, md.block_table, rows, lens, self.scale,
                                      md.max_seq_len, precise=True)
-        return ops.latent_row_attention(qf, self.rows, md.block_table, rows, lens, self.scale, self.rank, md.max_seq_len)
+        return ops.latent_row_attention(qf, self.rows, md.block_table, rows, lens, self.scale, self.rank, md.max_seq_len,
+                                        self.window, self.sink, gate)
 
 
 class WindowBiasAttention(Attention):
@@ -314,12 +335,18 @@ class WindowBiasAttention(Attention):
     ``i - j < window`` or ``j < keep_first``; its score is ``cap(q.k * scale) - bias_scale[h] * ln(1 +
     bias_rate[h] * (i - j))``.  The caches are key rows ``[blocks, Hkv, block, dim]`` and values with eight keys side
     by side per channel, ``[blocks, Hkv, block / 8, vdim, 8]``, written by ``ops.conv_norm_cache`` (this layer's callers convolve and normalise q / k / v
-    first); scores, softmax and the weighted sum of values are fp32 in every dtype."""
+    first); scores, softmax and the weighted sum of values are fp32 in every dtype.  ``chunk > 0`` replaces the window
+    by blocks of ``chunk`` positions counted from the sequence's start: a query sees the keys of its own block up to
+    itself (``window`` is then ``chunk``: no key further back is ever read, so the pages behind it are given back).
+    ``sink`` may be another instance's parameter (layers that run several times over one set of weights)."""
     row_cache = True
 
     def __init__(self, num_heads: int, dim: int, vdim: int, num_kv_heads: int, scale: float, layer_idx: int,
                  window: int = 0, keep_first: int = 0, softcap: Optional[float] = None, distance_bias: bool = True,
-                 sink: bool = True):
+                 sink=True, chunk: int = 0):
+        self.chunk = int(chunk or 0)
+        if self.chunk:
+            window, keep_first = self.chunk, 0
         super().__init__(num_heads, dim, num_kv_heads, scale, layer_idx, sliding_window=window, softcap=softcap)
         self.vdim = vdim
         self.keep_first = int(keep_first or 0) if self.window else 0
@@ -327,7 +354,10 @@ class WindowBiasAttention(Attention):
         # (fp32 whatever the model dtype: they enter the scores directly)
         self.bias_scale = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if distance_bias else None
         self.bias_rate = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if distance_bias else None
-        self.sink = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if sink else None
+        if isinstance(sink, nn.Parameter):
+            self.sink = sink
+        else:
+            self.sink = nn.Parameter(torch.zeros(num_heads, dtype=f32), requires_grad=False) if sink else None
 
     def kv_cache_shapes(self, num_blocks: int, block_size: int):
         if block_size % 8:
@@ -357,12 +387,12 @@ class WindowBiasAttention(Attention):
         if nd > 0:            # one row per sequence: the waves of a block share its keys
             ops.window_bias_attention(q[:nd], self.k_cache, self.v_cache, md.block_table[:nb], md.query_start_loc[:nb + 1],
                                       md.seq_lens[:nb], None, pos[:nd], *common,
-                                      None if gate is None else gate[:nd], 1, out=out[:nd])
+                                      None if gate is None else gate[:nd], 1, out=out[:nd], chunk=self.chunk)
         if md.num_prefills > 0:
             ops.window_bias_attention(q[nd:], self.k_cache, self.v_cache, md.block_table[nb:],
                                       md.prefill_query_start_loc, md.seq_lens[nb:], md.prefill_token_rows(pos), pos[nd:],
                                       *common, None if gate is None else gate[nd:], md.max_prefill_query_len,
-                                      out=out[nd:])
+                                      out=out[nd:], chunk=self.chunk)
         return out.view(t, self.num_heads * self.vdim)
 
 
@@ -382,6 +412,27 @@ class ScalarRMSNorm(nn.Module):
     def residual_add(self, y: torch.Tensor, residual: torch.Tensor, then: Optional["ScalarRMSNorm"] = None):
         return ops.scalar_norm_residual(y, self.weight, residual, None if then is None else then.weight, self.eps,
                                         self.dtype)
+
+
+class ResidualRMSNorm(nn.Module):
+    """RMS norm over an fp32 residual stream in fp32 arithmetic, with fp32 gains ``offset + weight`` (``offset`` 1: a
+    weight stored around zero).  ``forward`` returns the model dtype (the input of a projection); ``add`` folds one or
+    two sublayer outputs into the stream and hands back the normed sum in the same launch; ``after`` does so for an
+    output that is itself RMS-normed with ``post_weight`` before it joins the stream."""
+
+    def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, offset: float = 0.0):
+        super().__init__()
+        self.weight = nn.Parameter(torch.zeros(hidden_size, dtype=torch.float32), requires_grad=False)
+        self.eps, self.dtype, self.offset = eps, dtype, float(offset)
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return ops.rms_norm_to(x, self.weight, self.eps, out_dtype or self.dtype, self.offset)
+
+    def add(self, residual: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.add_rms_norm_to(residual, a, b, self.weight, self.eps, self.dtype, self.offset)
+
+    def after(self, y: torch.Tensor, post_weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        return ops.norm_add_norm(y, post_weight, residual, self.weight, self.eps, self.dtype, self.offset)
 
 
 class RMSNorm(nn.Module):

@@ -1,4 +1,4 @@
-"""Linear attention with a decay per head and a recurrent state per request.
+"""Linear attention with a recurrent state per request: a decay per head, or the gated delta rule.
 
 Per head ``S_t = decay[h] * S_(t-1) + k_t v_t^T`` and ``o_t = S_t^T q_t``: no softmax, no cache that grows with the
 sequence.  What a request carries from token to token is the ``dim x vdim`` matrix ``S`` of every head, in fp32, one
@@ -50,3 +50,32 @@ class DecayLinearAttention(nn.Module):
         return ops.decay_linear_attention(x, self.num_heads, self.dim, self.vdim, self.decay, self.state,
                                           md.state_slots, md.query_start_loc, md.seq_lens, self.activation,
                                           md.max_query_len)
+
+
+class GatedDeltaRule(nn.Module):
+    """The gated delta rule: per value head a ``dim x vdim`` fp32 state with
+    ``S <- g * S`` (one decay per key channel, by rows), ``u = b (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q``, on
+    unit-length q and k (q times ``dim^-0.5``), ``b = sigmoid(beta)`` and ``g = exp(-exp(a_log[h]) * softplus(dt +
+    dt_bias))``.  ``heads`` value heads share ``qk_heads`` query / key heads in runs of neighbours.  The state tensors
+    are ``layers.short_conv.SlotState`` objects the caller owns (one per run of the layer); ``forward`` reads
+    ``[q | k | v]`` from the leading columns of ``x`` and returns the fp32 heads ``[T, heads * vdim]`` side by side."""
+
+    def __init__(self, heads: int, qk_heads: int, dim: int, vdim: int, layer_idx: int, norm_eps: float = 1e-6):
+        super().__init__()
+        if heads % qk_heads:
+            raise ValueError(f"layer {layer_idx}: {heads} value heads do not divide over {qk_heads} query / key heads")
+        self.heads, self.qk_heads, self.dim, self.vdim = heads, qk_heads, dim, vdim
+        self.layer_idx, self.norm_eps = layer_idx, float(norm_eps)
+        self.a_log = nn.Parameter(torch.zeros(heads, dtype=torch.float32), requires_grad=False)
+        self.dt_bias = nn.Parameter(torch.zeros(heads * dim, dtype=torch.float32), requires_grad=False)
+
+    def per_slot_shape(self) -> Tuple[int, int, int]:
+        return (self.heads, self.dim, self.vdim)
+
+    def forward(self, x: torch.Tensor, beta: torch.Tensor, dt: torch.Tensor, state: Optional[torch.Tensor]) -> torch.Tensor:
+        md = get_forward_context().attn_metadata
+        if md is None or state is None:   # memory-profiling pass: no state bound
+            return x.new_zeros((x.shape[0], self.heads * self.vdim), dtype=torch.float32)
+        return ops.gated_delta_rule(x, self.heads, self.qk_heads, self.dim, self.vdim, beta, dt, self.dt_bias,
+                                    self.a_log, state, md.state_slots, md.query_start_loc, md.seq_lens, self.norm_eps,
+                                    md.max_query_len)

@@ -500,3 +500,98 @@ class GroupedIdentityMoE(FusedMoE):
             shared, gate = self.shared(x), self.shared_gate(x)
         return ops.expert_epilogue(out, x, topw if self.identity else None, topi if self.identity else None,
                                    self.real_experts, shared, gate)
+
+
+class BiasedTopKMoE(FusedMoE):
+    """Routed experts of the plain form ``down(act(up(x)))`` (no gate projection, no biases) behind a router with a
+    bias: the ``top_k`` largest of ``router(x) + bias`` are chosen and weighted by the softmax over just those.
+
+    The router is fp32 (product and bias).  On the GPU in 16-bit types the experts run as two grouped GEMMs over
+    expert-sorted rows, their reduction dimensions zero-padded to the kernels' 128-deep tiles; elsewhere (fp32, CPU)
+    one after the other on the library GEMM.  ``activation``: ``"gelu"`` (exact) or ``"gelu_tanh"``."""
+    custom_routing = True
+
+    def __init__(self, hidden: int, inter: int, num_experts: int, top_k: int, dtype: torch.dtype,
+                 activation: str = "gelu"):
+        super().__init__(hidden, inter, num_experts, top_k, True, dtype, expert_parallel=False, allocate_experts=False)
+        if self.tp > 1:
+            raise NotImplementedError("BiasedTopKMoE runs unsharded")
+        if not 1 <= top_k <= num_experts:
+            raise ValueError(f"top {top_k} of {num_experts} experts")
+        if activation not in ("gelu", "gelu_tanh"):
+            raise ValueError(f"unsupported expert activation {activation!r}")
+        self.quant = None
+        self.tanh = activation == "gelu_tanh"
+        self.gate = ReplicatedLinear(hidden, num_experts, False, dtype, quant=False)
+        self.gate_bias = nn.Parameter(torch.zeros(num_experts, dtype=torch.float32), requires_grad=False)
+        self.h_pad, self.i_pad = _ceil128(hidden), _ceil128(inter)
+        self.w1 = nn.Parameter(torch.zeros(num_experts, self.i_pad, self.h_pad, dtype=dtype), requires_grad=False)
+        self.w2 = nn.Parameter(torch.zeros(num_experts, hidden, self.i_pad, dtype=dtype), requires_grad=False)
+        self.w1.weight_loader = self._load_w1
+        self.w2.weight_loader = self._load_w2
+
+    def _load_w1(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        param.data[int(shard_id)].zero_()          # (the padding included: the loader poisons fresh parameters)
+        param.data[int(shard_id), :self.inter, :self.hidden].copy_(materialize(w))
+
+    def _load_w2(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        param.data[int(shard_id)].zero_()
+        param.data[int(shard_id), :, :self.inter].copy_(materialize(w))
+
+    def router_logits(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.linear_f32(x, self.gate.weight) + self.gate_bias
+
+    def route(self, logits: torch.Tensor):
+        val, topi = logits.float().topk(self.top_k, dim=-1)
+        return torch.softmax(val, dim=-1), topi
+
+    def _pad(self, x: torch.Tensor) -> torch.Tensor:
+        return x if self.h_pad == self.hidden else F.pad(x, (0, self.h_pad - self.hidden))
+
+    def _expert_mlp(self, e: int, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(ops.gelu(F.linear(self._pad(x), self.w1[e]), self.tanh), self.w2[e])
+
+    def _grouped_tile_rows(self, x: torch.Tensor) -> int:
+        if not (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and x.dim() == 2 and ops.hip_available()):
+            return 0
+        if self.num_experts > 512 or self.top_k > 16 or self.hidden % 16:
+            return 0
+        avg = x.shape[0] * self.top_k / max(1, self.num_experts)
+        if avg > envs.VDAMD_MOE_GROUPED_MAX_ROWS * 2 and not torch.cuda.is_current_stream_capturing():
+            return 0
+        for rows in (16, 32, 64, 128):
+            if avg <= rows:
+                return rows
+        return 128
+
+    def decode_capturable(self, dtype: torch.dtype) -> bool:
+        """Whether a decode step of this block runs without a host synchronisation (the grouped path)."""
+        return (dtype in (torch.bfloat16, torch.float16) and self.hidden % 16 == 0 and self.num_experts <= 512
+                and self.top_k <= 16)
+
+    def forward(self, x: torch.Tensor, reduce: bool = True, staged: bool = False, deferred: bool = False):
+        logits = self.router_logits(x)
+        tile_rows = self._grouped_tile_rows(x)
+        if tile_rows:
+            # (softmax over every output, the largest kept and renormalised: the softmax over the kept ones)
+            topw, topi = ops.moe_topk(logits, self.top_k, True)
+            src_row, inv, tiles = ops.moe_align_fused(topi, self.num_experts, tile_rows, 0, -1)
+            xs = self._pad(x).index_select(0, src_row)
+            h = ops.grouped_linear(xs, tiles, tile_rows, weight=self.w1)
+            y = ops.grouped_linear(ops.gelu(h, self.tanh), tiles, tile_rows, weight=self.w2)
+            return ops.moe_combine(y, topw, topi, inv, 0, -1)
+        topw, topi = self.route(logits)
+        acc = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        flat_e = topi.reshape(-1)
+        order = flat_e.argsort(stable=True)
+        counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()
+        tok = order // self.top_k
+        wts = topw.reshape(-1)[order]
+        start = 0
+        for eid, n in enumerate(counts):
+            if n:
+                seg = slice(start, start + n)
+                rows = tok[seg]
+                acc.index_add_(0, rows, self._expert_mlp(eid, x.index_select(0, rows)).float() * wts[seg].unsqueeze(1))
+            start += n
+        return acc.to(x.dtype)

@@ -56,3 +56,27 @@ class ShortConv(nn.Module):
 
     def bind_state(self, state: Optional[torch.Tensor]) -> None:
         self.state = state
+
+
+class SlotState:
+    """One per-request state tensor, ``[slots, *per_slot]``, of a layer whose weights live elsewhere: a layer that
+    runs several times in a forward pass over the same weights keeps one of these per run (the model lists them in
+    ``state_layers()``; the model runner allocates and binds them like a ``ShortConv``'s own state).
+    ``state_dtype`` None: the model dtype."""
+
+    def __init__(self, per_slot: Sequence[int], state_dtype: Optional[torch.dtype] = None):
+        self.per_slot = tuple(int(n) for n in per_slot)
+        self.state_dtype = state_dtype
+        self.state: Optional[torch.Tensor] = None
+
+    def state_shape(self, num_slots: int) -> Tuple[int, ...]:
+        return (num_slots,) + self.per_slot
+
+    def state_values_per_slot(self) -> int:
+        n = 1
+        for d in self.per_slot:
+            n *= d
+        return n
+
+    def bind_state(self, state: Optional[torch.Tensor]) -> None:
+        self.state = state

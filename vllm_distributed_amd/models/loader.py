@@ -54,6 +54,9 @@ def _weight_shapes(c: dict, arch: str) -> Dict[str, Tuple[int, ...]]:
     if arch in ("KabapelForCausalLM", "Kabapel"):
         from .kabapel import weight_shapes
         return weight_shapes(c)
+    if arch in ("GosizenForCausalLM", "Gosizen"):
+        from .gosizen import weight_shapes
+        return weight_shapes(c)
     if arch == "MedusaModel":
         h = c["hidden_size"]
         out = {}
@@ -463,6 +466,10 @@ def dummy_weights_iterator(mc: ModelConfig, device: torch.device,
             from .kabapel import random_weight
             yield name, random_weight(name, shape, gen, device, dtype)
             continue
+        if mc.architecture in ("GosizenForCausalLM", "Gosizen"):
+            from .gosizen import random_weight
+            yield name, random_weight(name, shape, gen, device, dtype)
+            continue
         if awq and _QUANTIZED_LINEAR.search(name) and shape[1] % g == 0 and shape[0] % 8 == 0:
             out_f, in_f = shape
             base = name[:-len(".weight")]
@@ -567,6 +574,20 @@ def _dequantize_stream(weights: Iterable[Tuple[str, torch.Tensor]], dtype: torch
                 break
         else:
             yield name, w
+
+
+def checkpoint_tensor_shapes(path: Optional[str]) -> Dict[str, Tuple[int, ...]]:
+    """Names and shapes of the tensors in a checkpoint directory's safetensors files (headers only; empty when there
+    is no such file): for a family whose config leaves a size to the shape of a tensor."""
+    if not path or not os.path.isdir(path):
+        return {}
+    from safetensors import safe_open
+    out: Dict[str, Tuple[int, ...]] = {}
+    for fn in sorted(glob.glob(os.path.join(path, "*.safetensors"))):
+        with safe_open(fn, framework="pt", device="cpu") as f:
+            for name in f.keys():
+                out[name] = tuple(f.get_slice(name).get_shape())
+    return out
 
 
 def safetensors_weights_iterator(path: str, dtype: torch.dtype,

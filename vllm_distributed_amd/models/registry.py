@@ -71,6 +71,10 @@ _MODELS: Dict[str, Tuple[str, str]] = {
     # rows; grouped routing with identity experts
     "KabapelForCausalLM": ("kabapel", "KabapelForCausalLM"),
     "Kabapel": ("kabapel", "KabapelForCausalLM"),
+    # fp32 residual stream; mixer and feed-forward side by side on one normed input; windowed latent attention,
+    # chunked attention over convolved keys beside the gated delta rule; a block of layers that runs several times
+    "GosizenForCausalLM": ("gosizen", "GosizenForCausalLM"),
+    "Gosizen": ("gosizen", "GosizenForCausalLM"),
     # draft heads of speculative decoding (never a served model by themselves; worker/draft_model.py)
     "EagleLlamaForCausalLM": ("spec_heads", "EagleLlamaForCausalLM"),
     "Eagle3LlamaForCausalLM": ("spec_heads", "Eagle3LlamaForCausalLM"),
@@ -82,7 +86,8 @@ _MODELS: Dict[str, Tuple[str, str]] = {
 
 # architectures whose layers keep per-request state besides the KV cache (convolution tails, recurrences): a cached
 # prefix's blocks do not bring that state back, so prefix reuse is off for them
-_KEEPS_REQUEST_STATE = {"TavulixForCausalLM", "Tavulix", "KabapelForCausalLM", "Kabapel"}
+_KEEPS_REQUEST_STATE = {"TavulixForCausalLM", "Tavulix", "KabapelForCausalLM", "Kabapel", "GosizenForCausalLM",
+                        "Gosizen"}
 
 
 def keeps_request_state(arch: str) -> bool:

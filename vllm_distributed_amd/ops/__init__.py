@@ -650,31 +650,33 @@ def poly_norm(z, coef, eps: float):
 
 def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions, num_heads: int,
                     num_kv_heads: int, dim: int, vdim: int, q_norm, k_norm, eps: float, v_first, v_lambda,
-                    keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True):
+                    keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True, inv_freq=None):
     """``conv_weight`` is tap-major, ``[taps, C]``.  Short convolution (with per-request state) + per-head q / k norm + value mixing + cache write over a fused
     projection; see ``torch_ref.conv_norm_cache``.  ``token_seq`` (None: row ``t`` belongs to sequence ``t``) and
-    ``positions`` tell the kernel which sequence and position each row has."""
+    ``positions`` tell the kernel which sequence and position each row has.  ``q_norm`` / ``k_norm`` None: no head
+    norm; ``inv_freq``: q and k heads are rotated (pairs half a rotation width apart) after the convolution."""
     if _use_hip(x):
         return _hip.conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions,
                                     num_heads, num_kv_heads, dim, vdim, q_norm, k_norm, eps, v_first, v_lambda,
-                                    keep_v, k_cache, v_cache, slot_mapping, has_prefill)
+                                    keep_v, k_cache, v_cache, slot_mapping, has_prefill, inv_freq)
     return torch_ref.conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, num_heads,
                                      num_kv_heads, dim, vdim, q_norm, k_norm, eps, v_first, v_lambda, keep_v,
-                                     k_cache, v_cache, slot_mapping)
+                                     k_cache, v_cache, slot_mapping, inv_freq, positions)
 
 
 def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
                           scale: float, softcap: float, window: int, keep_first: int, bias_scale, bias_rate, sinks,
-                          gate, max_query_len: int = 0, out=None):
-    """Attention over row caches with a window that keeps the first keys, a logarithmic distance bias, a sink in
-    the denominator and an output gate; see ``torch_ref.window_bias_attention``."""
+                          gate, max_query_len: int = 0, out=None, chunk: int = 0):
+    """Attention over row caches with a window that keeps the first keys (or, ``chunk > 0``, a mask of blocks of
+    ``chunk`` positions), a logarithmic distance bias, a sink in the denominator and an output gate; see
+    ``torch_ref.window_bias_attention``."""
     if _use_hip(q):
         attention_calls["hip"] += 1
         return _hip.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq,
                                           positions, scale, softcap, window, keep_first, bias_scale, bias_rate, sinks,
-                                          gate, max_query_len, out)
+                                          gate, max_query_len, out, chunk)
     res = torch_ref.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, scale,
-                                          softcap, window, keep_first, bias_scale, bias_rate, sinks, gate)
+                                          softcap, window, keep_first, bias_scale, bias_rate, sinks, gate, chunk)
     if out is not None:
         out.copy_(res)
         return out
@@ -714,10 +716,12 @@ def decay_linear_attention(x, num_heads: int, dim: int, vdim: int, decay, state,
     return torch_ref.decay_linear_attention(x, num_heads, dim, vdim, decay, state, slots, query_start_loc, seq_lens, silu)
 
 
-def gated_rms_norm(o, weight, gate, eps: float, out_dtype):
+def gated_rms_norm(o, weight, gate, eps: float, out_dtype, group: int = 0, scale: float = 1.0, out=None):
+    """RMS norm of fp32 rows (whole rows, or runs of ``group`` values sharing ``weight[group]``) times
+    ``sigmoid(gate) * scale``; ``out``: a view with strided rows that receives the result."""
     if _use_hip(o):
-        return _hip.gated_rms_norm(o, weight, gate, eps, out_dtype)
-    return torch_ref.gated_rms_norm(o, weight, gate, eps, out_dtype)
+        return _hip.gated_rms_norm(o, weight, gate, eps, out_dtype, group, scale, out)
+    return torch_ref.gated_rms_norm(o, weight, gate, eps, out_dtype, group, scale, out)
 
 
 def clamped_glu(h, limit: float, alpha: float):
@@ -733,19 +737,21 @@ def relu_squared(x):
 
 
 def latent_prep(q, nope: int, q_lat, latent, norm_weight, eps: float, inv_freq, rot_scale: float, positions, cache,
-                slot_mapping, fragments=None):
+                slot_mapping, fragments=None, interleaved: bool = False):
     if _use_hip(q):
         return _hip.latent_prep(q, nope, q_lat, latent, norm_weight, eps, inv_freq, rot_scale, positions, cache,
-                                slot_mapping, fragments)
+                                slot_mapping, fragments, interleaved)
     return torch_ref.latent_prep(q, nope, q_lat, latent, norm_weight, eps, inv_freq, rot_scale, positions, cache,
-                                 slot_mapping, fragments)
+                                 slot_mapping, fragments, interleaved)
 
 
-def latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale: float, rank: int, max_seq_len: int = 0):
+def latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale: float, rank: int, max_seq_len: int = 0,
+                         window: int = 0, sinks=None, gate=None):
     if _use_hip(q):
         attention_calls["hip"] += 1
-        return _hip.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank, max_seq_len)
-    return torch_ref.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank)
+        return _hip.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank, max_seq_len,
+                                         window, sinks, gate)
+    return torch_ref.latent_row_attention(q, cache, block_table, token_seq, seq_lens, scale, rank, window, sinks, gate)
 
 
 def expert_epilogue(routed, x, topw, topi, real_experts: int, shared, gate):
@@ -754,3 +760,70 @@ def expert_epilogue(routed, x, topw, topi, real_experts: int, shared, gate):
     if _use_hip(routed) and (topi is None or topi.dtype == torch.int32):
         return _hip.expert_epilogue(routed, x, topw, topi, real_experts, shared, gate)
     return torch_ref.expert_epilogue(routed, x, topw, topi, real_experts, shared, gate)
+
+
+# ------------------------------------------------ fp32 residual stream with offset RMS norms, side inputs per token,
+# ------------------------------------------------ convolutions with activation, the gated delta rule
+def rms_norm_to(x, weight, eps: float, out_dtype, offset: float = 0.0):
+    """RMS norm in fp32 arithmetic of rows of any float type with fp32 gains ``offset + weight``; see
+    ``torch_ref.rms_norm_to``."""
+    if _use_hip(x):
+        return _hip.rms_norm_to(x, weight, eps, out_dtype, offset)
+    return torch_ref.rms_norm_to(x, weight, eps, out_dtype, offset)
+
+
+def add_rms_norm_to(residual, a, b, weight, eps: float, out_dtype, offset: float = 0.0, normed: bool = True):
+    """``residual += a + b`` on the fp32 residual stream and the RMS norm of the sum (or the sum itself) in
+    ``out_dtype``: one launch."""
+    if _use_hip(residual):
+        return _hip.add_rms_norm_to(residual, a, b, weight, eps, out_dtype, offset, normed)
+    return torch_ref.add_rms_norm_to(residual, a, b, weight, eps, out_dtype, offset, normed)
+
+
+def norm_add_norm(y, post_weight, residual, next_weight, eps: float, out_dtype, next_offset: float = 0.0,
+                  next_normed: bool = True):
+    """``residual += rms_norm(y) * post_weight`` on the fp32 residual stream and the RMS norm of the sum (or the sum
+    itself) in ``out_dtype``: one launch."""
+    if _use_hip(y):
+        return _hip.norm_add_norm(y, post_weight, residual, next_weight, eps, out_dtype, next_offset, next_normed)
+    return torch_ref.norm_add_norm(y, post_weight, residual, next_weight, eps, out_dtype, next_offset, next_normed)
+
+
+def gelu_mul_rows(g, table, ids, col: int):
+    if _use_hip(g):
+        return _hip.gelu_mul_rows(g, table, ids, col)
+    return torch_ref.gelu_mul_rows(g, table, ids, col)
+
+
+def sigmoid_mul(o, gate, scale: float = 1.0, out=None):
+    if _use_hip(o):
+        return _hip.sigmoid_mul(o, gate, scale, out)
+    return torch_ref.sigmoid_mul(o, gate, scale, out)
+
+
+def gelu(x, tanh: bool):
+    """GELU (the tanh form or the exact one) in fp32 arithmetic, in ``x``'s dtype."""
+    if _use_hip(x):
+        return _hip.gelu(x, tanh)
+    return torch.nn.functional.gelu(x.float(), approximate="tanh" if tanh else "none").to(x.dtype)
+
+
+def short_conv_act(x, channels: int, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions,
+                   silu: bool, has_prefill: bool = True):
+    """Causal convolution over time (tap-major ``conv_weight[taps, channels]``, per-request state) of the first
+    ``channels`` columns of a fused projection, through SiLU when asked; see ``torch_ref.short_conv_act``."""
+    if _use_hip(x):
+        return _hip.short_conv_act(x, channels, conv_weight, state, slots, query_start_loc, seq_lens, token_seq,
+                                   positions, silu, has_prefill)
+    return torch_ref.short_conv_act(x, channels, conv_weight, state, slots, query_start_loc, seq_lens, silu)
+
+
+def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, beta, dt, dt_bias, a_log, state,
+                     slots, query_start_loc, seq_lens, norm_eps: float = 1e-6, max_query_len: int = 0):
+    """The gated delta rule with a decay per head and key channel and a per-request fp32 state; see
+    ``torch_ref.gated_delta_rule``."""
+    if _use_hip(x):
+        return _hip.gated_delta_rule(x, num_heads, num_qk_heads, dim, vdim, beta, dt, dt_bias, a_log, state, slots,
+                                     query_start_loc, seq_lens, norm_eps, max_query_len)
+    return torch_ref.gated_delta_rule(x, num_heads, num_qk_heads, dim, vdim, beta, dt, dt_bias, a_log, state, slots,
+                                      query_start_loc, seq_lens, norm_eps)

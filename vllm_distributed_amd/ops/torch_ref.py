@@ -502,10 +502,13 @@ def conv_norm_cache(x: torch.Tensor, conv_weight: torch.Tensor, state: torch.Ten
                     query_start_loc: torch.Tensor, seq_lens: torch.Tensor, num_heads: int, num_kv_heads: int,
                     dim: int, vdim: int, q_norm: torch.Tensor, k_norm: torch.Tensor, eps: float,
                     v_first: Optional[torch.Tensor], v_lambda: Optional[torch.Tensor], keep_v: bool,
-                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slot_mapping: torch.Tensor):
+                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slot_mapping: torch.Tensor,
+                    inv_freq: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None):
     """Everything between the fused projection and the attention of a layer whose q / k / v pass through a short
     convolution: ``x[T, C_x]`` holds ``[q | k | v | ...]`` (columns past the three are not touched);
-    ``short_conv`` over the first ``C`` columns, RMS norm of each q and k head with the ``[dim]`` weights,
+    ``short_conv`` over the first ``C`` columns, RMS norm of each q and k head with the ``[dim]`` weights (skipped when
+    ``q_norm`` is None), then, with ``inv_freq``, the rotation of each q and k head's first ``2 * len(inv_freq)``
+    values by ``positions`` (value ``i`` paired with value ``i + len(inv_freq)``),
     ``v <- (1 - v_lambda) v + v_lambda v_first`` when ``v_first[T, Hkv * vdim]`` (fp32) is given, k and the mixed
     v into the row caches ``[blocks, Hkv, block, dim | vdim]`` at ``slot_mapping``.  Returns ``(q[T, Hq, dim]``
     in ``x``'s dtype, the unmixed fp32 ``v`` if ``keep_v`` else None``)``."""
@@ -515,10 +518,16 @@ def conv_norm_cache(x: torch.Tensor, conv_weight: torch.Tensor, state: torch.Ten
     y = short_conv(x[:, :c], conv_weight, state, slots, query_start_loc, seq_lens)
 
     def head_norm(u, w):
+        if w is None:
+            return u
         return u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()
 
-    q = head_norm(y[:, :qs].reshape(t, num_heads, dim), q_norm).to(x.dtype)
+    q = head_norm(y[:, :qs].reshape(t, num_heads, dim), q_norm)
     k = head_norm(y[:, qs:qs + ks].reshape(t, num_kv_heads, dim), k_norm)
+    if inv_freq is not None and inv_freq.numel():
+        q = rotate_pairs_first(q, positions[:t], inv_freq, 1.0)
+        k = rotate_pairs_first(k, positions[:t], inv_freq, 1.0)
+    q = q.to(x.dtype)
     v = y[:, qs + ks:].reshape(t, num_kv_heads, vdim)
     kept = v.reshape(t, vs).clone() if keep_v else None
     if v_first is not None:
@@ -538,11 +547,12 @@ def window_bias_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                           query_start_loc: torch.Tensor, seq_lens: torch.Tensor, scale: float, softcap: float,
                           window: int, keep_first: int, bias_scale: Optional[torch.Tensor],
                           bias_rate: Optional[torch.Tensor], sinks: Optional[torch.Tensor],
-                          gate: Optional[torch.Tensor]) -> torch.Tensor:
+                          gate: Optional[torch.Tensor], chunk: int = 0) -> torch.Tensor:
     """Causal attention over ``k_cache[blocks, Hkv, block, D]`` (key rows) and ``v_cache[blocks, Hkv, block / 8, Dv,
     8]`` (eight keys side by side per channel).
     A query at position ``i`` sees key ``j <= i`` when ``i - j < window`` (``window`` 0: no limit) or
-    ``j < keep_first``.  ``score = q.k * scale``, squashed to ``softcap * tanh(score / softcap)`` when
+    ``j < keep_first``; with ``chunk > 0`` it sees ``j <= i`` only inside its own block of ``chunk`` positions
+    counted from the sequence's start (``i // chunk == j // chunk``).  ``score = q.k * scale``, squashed to ``softcap * tanh(score / softcap)`` when
     ``softcap > 0``, minus ``bias_scale[h] * ln(1 + bias_rate[h] * (i - j))``; ``sinks[h]`` adds ``exp(sinks[h])``
     to the softmax denominator; ``gate[T, Hq]`` multiplies head ``h``'s output by ``sigmoid(gate[t, h])``.
     fp32 arithmetic; returns ``[T, Hq, Dv]`` in ``q``'s dtype."""
@@ -571,6 +581,8 @@ def window_bias_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         seen = kpos <= qpos
         if window > 0:
             seen = seen & (((qpos - kpos) < window) | (kpos < keep_first))
+        if chunk > 0:
+            seen = seen & (torch.div(qpos, chunk, rounding_mode="floor") == torch.div(kpos, chunk, rounding_mode="floor"))
         sc = sc.masked_fill(~seen, float("-inf"))
         if sinks is not None:
             col = sinks.float().view(-1, 1, 1).expand(hq, ql, 1)
@@ -641,11 +653,22 @@ def decay_linear_attention(x: torch.Tensor, num_heads: int, dim: int, vdim: int,
 
 
 def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps: float,
-                   out_dtype: torch.dtype) -> torch.Tensor:
-    """``o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate)`` over whole rows, fp32 arithmetic."""
+                   out_dtype: torch.dtype, group: int = 0, scale: float = 1.0,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate) * scale`` in fp32 arithmetic, the mean over whole rows or,
+    with ``group > 0``, over each run of ``group`` values (``weight[group]`` then serves every run).  ``out``: a
+    ``[T, N]`` view (rows may be strided) that receives the result."""
     of = o.float()
-    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
-    return (y * torch.sigmoid(gate.float())).to(out_dtype)
+    if group > 0:
+        g = of.unflatten(-1, (-1, group))
+        y = (g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).flatten(-2)
+    else:
+        y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    y = y * torch.sigmoid(gate.float()) * scale
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y.to(out_dtype)
 
 
 def clamped_glu(h: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
@@ -668,25 +691,39 @@ def rotate_half_first(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.
     return torch.cat([u * cos - v * sin, v * cos + u * sin, x[..., 2 * half:]], dim=-1)
 
 
+def rotate_pairs_first(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rot_scale: float,
+                       interleaved: bool = False) -> torch.Tensor:
+    """``rotate_half_first`` with a choice of pairing: ``interleaved`` pairs value ``2i`` with value ``2i + 1``."""
+    if not interleaved:
+        return rotate_half_first(x.float(), positions, inv_freq, rot_scale)
+    half = inv_freq.numel()
+    xf = x.float()
+    a = positions.float().view(-1, *([1] * (x.dim() - 1))) * inv_freq.float()
+    cos, sin = torch.cos(a) * rot_scale, torch.sin(a) * rot_scale
+    u, v = xf[..., 0:2 * half:2], xf[..., 1:2 * half:2]
+    rot = torch.stack([u * cos - v * sin, v * cos + u * sin], dim=-1).flatten(-2)
+    return torch.cat([rot, xf[..., 2 * half:]], dim=-1)
+
+
 def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
                 norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor, rot_scale: float,
                 positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
-                fragments: Optional[torch.Tensor] = None) -> torch.Tensor:
+                fragments: Optional[torch.Tensor] = None, interleaved: bool = False) -> torch.Tensor:
     """Between the projections and the attention of a layer whose keys and values are one shared latent row per
     token.  ``q[T, H, nope + rope]``, ``q_lat[H, T, rank]`` (the unrotated query part already multiplied into the
     latent space): returns ``[T, H, rank + rope] = [q_lat | rotated q[..., nope:]]``.  With ``latent[T, rank + rope]``
     the row ``[RMS norm of the first rank values * norm_weight | rotated last rope values]`` goes into
     ``cache[blocks, 1, block, rank + rope]`` at ``slot_mapping`` (a layer that reads another layer's rows passes
     None), and its first ``rank`` values also into ``fragments`` (the V^T fragment cache, see ``v_cache_shape``) when
-    the layer keeps one.  Norm and rotation in fp32."""
+    the layer keeps one.  Norm and rotation in fp32; ``interleaved`` pairs neighbouring values in the rotation."""
     t = q.shape[0]
-    q_rot = rotate_half_first(q[..., nope:].float(), positions[:t], inv_freq, rot_scale)
+    q_rot = rotate_pairs_first(q[..., nope:], positions[:t], inv_freq, rot_scale, interleaved)
     out = torch.cat([q_lat.transpose(0, 1).float(), q_rot], dim=-1).to(q.dtype)
     if latent is not None and cache is not None and slot_mapping is not None:
         rank = q_lat.shape[2]
         c = latent[:, :rank].float()
         c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
-        kr = rotate_half_first(latent[:, rank:].float(), positions[:t], inv_freq, rot_scale)
+        kr = rotate_pairs_first(latent[:, rank:], positions[:t], inv_freq, rot_scale, interleaved)
         row = torch.cat([c, kr], dim=-1).to(cache.dtype)
         bs = cache.shape[2]
         valid = slot_mapping[:t] >= 0
@@ -699,10 +736,14 @@ def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optiona
 
 
 def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
-                         token_seq: Optional[torch.Tensor], seq_lens: torch.Tensor, scale: float, rank: int) -> torch.Tensor:
+                         token_seq: Optional[torch.Tensor], seq_lens: torch.Tensor, scale: float, rank: int,
+                         window: int = 0, sinks: Optional[torch.Tensor] = None,
+                         gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``q[T, H, DK]`` against ``cache[blocks, 1, block, DK]``: token ``t`` reads block-table row ``token_seq[t]``
-    (``t`` itself when None) and sees keys ``0 .. seq_lens[t] - 1``; a key row's first ``rank`` values are also its
-    value.  Scores, softmax and the weighted sum in fp32; returns ``[T, H, rank]`` in ``q``'s dtype."""
+    (``t`` itself when None) and sees keys ``0 .. seq_lens[t] - 1``, with ``window > 0`` only the last ``window`` of
+    them; a key row's first ``rank`` values are also its value.  ``sinks[H]`` adds ``exp(sinks[h])`` to head ``h``'s
+    softmax denominator; ``gate[T, H]`` multiplies head ``h``'s output by ``sigmoid(gate[t, h])``.  Scores, softmax and
+    the weighted sum in fp32; returns ``[T, H, rank]`` in ``q``'s dtype."""
     t, hq, dk = q.shape
     bs = cache.shape[2]
     res = torch.zeros((t, hq, rank), dtype=torch.float32, device=q.device)
@@ -713,12 +754,23 @@ def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torc
         n = int(lens[mine].max())
         if n == 0:
             continue
-        blocks = block_table[b, :(n + bs - 1) // bs].long()
-        keys = cache[blocks, 0].reshape(-1, dk)[:n].float()
+        first = max(int(lens[mine].min()) - window, 0) if window > 0 else 0      # (blocks before it may be gone)
+        blocks = block_table[b, first // bs:(n + bs - 1) // bs].long()
+        keys = cache[blocks, 0].reshape(-1, dk)[:n - first // bs * bs].float()
+        kpos = torch.arange(first // bs * bs, n, device=q.device)[None, None, :]
         s = torch.einsum("thd,nd->thn", q[mine].float(), keys) * scale
-        mask = torch.arange(n, device=q.device)[None, None, :] >= lens[mine][:, None, None]
-        p = torch.softmax(s.masked_fill(mask, float("-inf")), dim=-1)
+        mask = kpos >= lens[mine][:, None, None]
+        if window > 0:
+            mask = mask | (kpos < lens[mine][:, None, None] - window)
+        s = s.masked_fill(mask, float("-inf"))
+        if sinks is not None:
+            col = sinks.float().view(1, hq, 1).expand(mine.numel(), hq, 1)
+            p = torch.softmax(torch.cat([s, col], dim=-1), dim=-1)[..., :-1]
+        else:
+            p = torch.softmax(s, dim=-1)
         res[mine] = torch.einsum("thn,nd->thd", p, keys[:, :rank])
+    if gate is not None:
+        res = res * torch.sigmoid(gate[:t].float()).unsqueeze(-1)
     return res.to(q.dtype)
 
 
@@ -733,3 +785,105 @@ def expert_epilogue(routed: torch.Tensor, x: torch.Tensor, topw: Optional[torch.
     if shared is not None:
         out = out + shared.float() * torch.sigmoid(gate.float().reshape(-1, 1))
     return out.to(routed.dtype)
+
+
+# ------------------------------------------------ fp32 residual stream with offset RMS norms, side inputs per token,
+# ------------------------------------------------ convolutions with activation, the gated delta rule
+def rms_norm_to(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+                offset: float = 0.0) -> torch.Tensor:
+    """``x / sqrt(mean(x^2) + eps) * (offset + weight)`` over the last dimension in fp32 arithmetic (``weight`` None:
+    no gain), result in ``out_dtype``."""
+    xf = x.float()
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * (weight.float() + offset)
+    return y.to(out_dtype)
+
+
+def add_rms_norm_to(residual: torch.Tensor, a: Optional[torch.Tensor], b: Optional[torch.Tensor],
+                    weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype, offset: float = 0.0,
+                    normed: bool = True) -> torch.Tensor:
+    """``residual += a + b`` in place on the fp32 residual stream (either may be None), then ``rms_norm_to`` of the
+    sum, or with ``normed`` False just the sum, in ``out_dtype``."""
+    if a is not None:
+        residual.add_(a.float() if b is None else a.float() + b.float())
+    if not normed:
+        return residual.to(out_dtype)
+    return rms_norm_to(residual, weight, eps, out_dtype, offset)
+
+
+def norm_add_norm(y: torch.Tensor, post_weight: torch.Tensor, residual: torch.Tensor,
+                  next_weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype, next_offset: float = 0.0,
+                  next_normed: bool = True) -> Optional[torch.Tensor]:
+    """``residual += rms_norm(y) * post_weight`` in place on the fp32 residual stream; then what
+    ``add_rms_norm_to(residual, None, None, next_weight, ...)`` returns."""
+    residual.add_(rms_norm_to(y, post_weight, eps, torch.float32))
+    if not next_normed:
+        return residual.to(out_dtype)
+    return rms_norm_to(residual, next_weight, eps, out_dtype, next_offset)
+
+
+def gelu_tanh_f(z: torch.Tensor) -> torch.Tensor:
+    return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+
+
+def gelu_mul_rows(g: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col: int) -> torch.Tensor:
+    """``gelu_tanh(g[T, n]) * table[ids, col : col + n]`` in fp32 arithmetic, result in ``g``'s dtype."""
+    n = g.shape[1]
+    return (gelu_tanh_f(g.float()) * table[ids.long(), col:col + n].float()).to(g.dtype)
+
+
+def sigmoid_mul(o: torch.Tensor, gate: torch.Tensor, scale: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``o * sigmoid(gate) * scale`` in fp32 arithmetic, in ``o``'s dtype; ``out``: a view that receives it."""
+    y = o.float() * torch.sigmoid(gate.float()) * scale
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y.to(o.dtype)
+
+
+def short_conv_act(x: torch.Tensor, channels: int, conv_weight: torch.Tensor, state: torch.Tensor, slots: torch.Tensor,
+                   query_start_loc: torch.Tensor, seq_lens: torch.Tensor, silu: bool) -> torch.Tensor:
+    """``short_conv`` over the first ``channels`` columns of ``x`` (the state moves on), through SiLU when ``silu``;
+    ``[T, channels]`` in ``x``'s dtype."""
+    y = short_conv(x[:, :channels], conv_weight, state, slots, query_start_loc, seq_lens)
+    return (F.silu(y) if silu else y).to(x.dtype)
+
+
+def gated_delta_rule(x: torch.Tensor, num_heads: int, num_qk_heads: int, dim: int, vdim: int, beta: torch.Tensor,
+                     dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor,
+                     slots: torch.Tensor, query_start_loc: torch.Tensor, seq_lens: torch.Tensor,
+                     norm_eps: float = 1e-6) -> torch.Tensor:
+    """The gated delta rule over the packed rows ``x[T, C]`` = ``[q (Hqk * dim) | k (Hqk * dim) | v (H * vdim)]``;
+    value head ``h`` reads q / k head ``h // (H / Hqk)``.  Per row: q and k become unit vectors
+    (``u / sqrt(sum(u^2) + norm_eps)``), q times ``dim^-0.5``; ``b = sigmoid(beta[t, h])``; one decay per head and
+    key channel ``g = exp(-exp(a_log[h]) * softplus(dt[t, h, :] + dt_bias[h, :]))``; then ``S <- g * S`` by rows,
+    ``u = b (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q``.  ``S`` is ``state[slots[i]]`` (``[slots, H, dim, vdim]``
+    fp32) for sequence ``i``, taken as zero when the rows start at position 0 whatever the slot held, and left holding
+    the state after the sequence's last row.  fp32 arithmetic; returns fp32 ``[T, H * vdim]``."""
+    t, h, g = x.shape[0], num_heads, num_qk_heads
+    qs = g * dim
+    xf = x[:, :2 * qs + h * vdim].float()
+    q = xf[:, :qs].reshape(t, g, dim)
+    k = xf[:, qs:2 * qs].reshape(t, g, dim)
+    q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + norm_eps) * dim ** -0.5
+    k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + norm_eps)
+    q, k = q.repeat_interleave(h // g, dim=1), k.repeat_interleave(h // g, dim=1)
+    v = xf[:, 2 * qs:].reshape(t, h, vdim)
+    b = torch.sigmoid(beta[:t].float())
+    decay = torch.exp(-torch.exp(a_log.float()).view(1, h, 1)
+                      * F.softplus(dt[:t].float().reshape(t, h, dim) + dt_bias.float().view(1, h, dim)))
+    out = torch.zeros((t, h, vdim), dtype=torch.float32, device=x.device)
+    qsl, sls, sl = query_start_loc.tolist(), seq_lens.tolist(), slots.tolist()
+    for i, n_ctx in enumerate(sls):
+        s, e = qsl[i], qsl[i + 1]
+        if e == s:
+            continue
+        st = state[sl[i]].float().clone() if n_ctx - (e - s) > 0 else torch.zeros_like(state[sl[i]], dtype=torch.float32)
+        for r in range(s, e):
+            st = decay[r].unsqueeze(2) * st
+            u = b[r].unsqueeze(1) * (v[r] - torch.einsum("hkv,hk->hv", st, k[r]))
+            st = st + k[r].unsqueeze(2) * u.unsqueeze(1)
+            out[r] = torch.einsum("hkv,hk->hv", st, q[r])
+        state[sl[i]] = st.to(state.dtype)
+    return out.reshape(t, h * vdim)
