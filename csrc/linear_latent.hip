@@ -10,7 +10,8 @@
 //                            one head's S for one sequence, in registers (up to 16 waves x dim/16 rows each), and walks
 //                            the sequence's rows in chunks staged through LDS: prompt portions and single decoded rows
 //                            are the same kernel (launches of decoded rows only take small workgroups)
-//   gated_rms_norm           o / sqrt(mean(o^2) + eps) * w * sigmoid(g)
+//   gated_rms_norm           o / sqrt(mean(o^2) + eps) * w * sigmoid(g) * scale, over whole rows or over runs of `group`
+//                            values (heads) that share w
 //   clamped_glu              min(g, L) sigmoid(alpha min(g, L)) (clamp(u, -L, L) + 1) over [g | u]
 //   relu_squared             max(x, 0)^2
 //   expert_epilogue          routed + x * (weights of the chosen identity experts) + shared * sigmoid(gate)
@@ -18,7 +19,8 @@
 //                            the query [q_lat | rotated q_rope] assembled; angles = position * frequency in fp32
 //   latent_row_attention     causal softmax attention of every head over the shared rows (value = a row's first
 //                            `rank` values): one wave per (token, head), a lane per key for the scores, lanes over
-//                            the value's columns for the weighted sum, online softmax; any sizes, any float type
+//                            the value's columns for the weighted sum, online softmax; any sizes, any float type;
+//                            optionally a sliding window, a sink per head in the denominator, a sigmoid gate per head
 #include "common.h"
 #include <math.h>
 #include <type_traits>
@@ -86,8 +88,9 @@ __global__ void layer_norm_kernel(TO* __restrict__ out, TX* __restrict__ x, long
 }
 
 template <typename TG, typename TO>
-__global__ void gated_rms_norm_kernel(TO* __restrict__ out, const float* __restrict__ o, const float* __restrict__ w,
-                                      const TG* __restrict__ gate, long gate_stride, float eps, int N) {
+__global__ void gated_rms_norm_kernel(TO* __restrict__ out, long out_stride, const float* __restrict__ o,
+                                      const float* __restrict__ w, const TG* __restrict__ gate, long gate_stride,
+                                      float eps, int N, float scale) {
   __shared__ float red[17];
   const long row = blockIdx.x;
   const float* orow = o + row * (long)N;
@@ -95,8 +98,29 @@ __global__ void gated_rms_norm_kernel(TO* __restrict__ out, const float* __restr
   float ss = 0.f;
   for (int i = threadIdx.x; i < N; i += blockDim.x) { const float f = orow[i]; ss += f * f; }
   const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)N + eps);
-  TO* dst = out + row * (long)N;
-  for (int i = threadIdx.x; i < N; i += blockDim.x) stf(dst + i, orow[i] * inv * w[i] * sigmoid_f(ldf(g + i)));
+  TO* dst = out + row * out_stride;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) stf(dst + i, orow[i] * inv * w[i] * sigmoid_f(ldf(g + i)) * scale);
+}
+
+// the norm over runs of `group` values (one head each) that share w[group]: a wave per run, rows x runs of work
+template <typename TG, typename TO>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(TO* __restrict__ out, long out_stride,
+                                                               const float* __restrict__ o, const float* __restrict__ w,
+                                                               const TG* __restrict__ gate, long gate_stride, float eps,
+                                                               int rows, int N, int group, float scale) {
+  const int lane = threadIdx.x & 63;
+  const int per_row = N / group;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= (long)rows * per_row) return;
+  const long row = unit / per_row;
+  const int c0 = (int)(unit - row * per_row) * group;
+  const float* orow = o + row * (long)N + c0;
+  float ss = 0.f;
+  for (int i = lane; i < group; i += 64) { const float f = orow[i]; ss += f * f; }
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)group + eps);
+  const TG* g = gate + row * gate_stride + c0;
+  TO* dst = out + row * out_stride + c0;
+  for (int i = lane; i < group; i += 64) stf(dst + i, orow[i] * inv * w[i] * sigmoid_f(ldf(g + i)) * scale);
 }
 
 // 16-bit gate and result, rows whose length and gate stride are multiples of 8: 16-byte accesses
@@ -330,7 +354,8 @@ __global__ void latent_prep_kernel(T* __restrict__ out, const T* __restrict__ q,
                                    long lat_st, const float* __restrict__ norm_w, float eps,
                                    const float* __restrict__ inv_freq, int half, float rs,
                                    const int* __restrict__ positions, T* __restrict__ cache, T* __restrict__ vfrag,
-                                   const int* __restrict__ slot_mapping, int H, int rank, int rope, int bs) {
+                                   const int* __restrict__ slot_mapping, int H, int rank, int rope, int bs,
+                                   int interleaved) {
   __shared__ float red[17];
   const long t = blockIdx.x;
   const int pos = positions[t];
@@ -345,10 +370,13 @@ __global__ void latent_prep_kernel(T* __restrict__ out, const T* __restrict__ q,
     const T* src = q + t * q_st + h * q_sh + nope;
     float val;
     if (j < 2 * half) {
-      const int p = j < half ? j : j - half;
+      // pair p: values (p, p + half), or neighbours (2p, 2p + 1)
+      const int p = interleaved ? j >> 1 : (j < half ? j : j - half);
+      const bool first = interleaved ? (j & 1) == 0 : j < half;
       float a, bb;
-      rotate_pair(ldf(src + p), ldf(src + p + half), pos, inv_freq[p], rs, a, bb);
-      val = j < half ? a : bb;
+      rotate_pair(ldf(src + (interleaved ? 2 * p : p)), ldf(src + (interleaved ? 2 * p + 1 : p + half)), pos,
+                  inv_freq[p], rs, a, bb);
+      val = first ? a : bb;
     } else {
       val = ldf(src + j);
     }
@@ -375,10 +403,12 @@ __global__ void latent_prep_kernel(T* __restrict__ out, const T* __restrict__ q,
   for (int j = threadIdx.x; j < rope; j += blockDim.x) {
     float val;
     if (j < 2 * half) {
-      const int p = j < half ? j : j - half;
+      const int p = interleaved ? j >> 1 : (j < half ? j : j - half);
+      const bool first = interleaved ? (j & 1) == 0 : j < half;
       float a, bb;
-      rotate_pair(ldf(lr + rank + p), ldf(lr + rank + p + half), pos, inv_freq[p], rs, a, bb);
-      val = j < half ? a : bb;
+      rotate_pair(ldf(lr + rank + (interleaved ? 2 * p : p)), ldf(lr + rank + (interleaved ? 2 * p + 1 : p + half)), pos,
+                  inv_freq[p], rs, a, bb);
+      val = first ? a : bb;
     } else {
       val = ldf(lr + rank + j);
     }
@@ -416,7 +446,7 @@ template <typename T, int NV>
 __global__ __launch_bounds__(256) void latent_row_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
     long bt_stride, const int* __restrict__ token_seq, const int* __restrict__ seq_lens, float scale, int H, int dk,
-    int rank, int bs) {
+    int rank, int bs, int window, const float* __restrict__ sinks, const T* __restrict__ gate, long gate_stride) {
   extern __shared__ float q_lds[];
   const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long t = blockIdx.x;
@@ -432,7 +462,9 @@ __global__ __launch_bounds__(256) void latent_row_attention_kernel(
   float o[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) o[i] = 0.f;
-  for (int j0 = 0; j0 < n; j0 += 64) {
+  // with a window only the last `window` keys are read (the pages before them may have gone back to the pool)
+  const int first = window > 0 ? max(n - window, 0) : 0;
+  for (int j0 = first; j0 < n; j0 += 64) {
     const int j = j0 + lane;
     const bool valid = j < n;
     long row = 0;
@@ -461,8 +493,17 @@ __global__ __launch_bounds__(256) void latent_row_attention_kernel(
       }
     }
   }
+  if (sinks != nullptr) {                        // exp(sink) joins the denominator, once, with no value
+    const float sk = sinks[h];
+    const float m_f = fmaxf(m, sk);
+    const float corr = expf(m - m_f);
+    l = l * corr + expf(sk - m_f);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) o[i] *= corr;
+  }
   T* orow = out + (t * H + h) * (long)rank;
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  float inv = l > 0.f ? 1.0f / l : 0.f;
+  if (gate != nullptr) inv *= sigmoid_f(ldf(gate + t * gate_stride + h));
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int dcol = lane + 64 * i;
@@ -507,12 +548,27 @@ VDAMD_API int vdamd_layer_norm_to(void* out, void* x, long x_stride, const void*
   return 0;
 }
 
-VDAMD_API int vdamd_gated_rms_norm(void* out, const float* o, const float* w, const void* gate, long gate_stride,
-                                   float eps, int rows, int N, int gate_dt, int out_dt, hipStream_t stream) {
+VDAMD_API int vdamd_gated_rms_norm(void* out, long out_stride, const float* o, const float* w, const void* gate,
+                                   long gate_stride, float eps, int rows, int N, int group, float scale, int gate_dt,
+                                   int out_dt, hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (N <= 0) return 1;
+  if (N <= 0 || group < 0 || (group > 0 && N % group) || out_stride < N) return 1;
   int inner = 0;
-  if (gate_dt != DT_F32 && gate_dt == out_dt && N % 8 == 0 && gate_stride % 8 == 0 && aligned16(gate) && aligned16(o) &&
+  if (group > 0) {
+    const long units = (long)rows * (N / group);
+    const int rc = by_dtype(gate_dt, [&](auto* tg) {
+      using TG = std::remove_pointer_t<decltype(tg)>;
+      inner = by_dtype(out_dt, [&](auto* to) {
+        using TO = std::remove_pointer_t<decltype(to)>;
+        hipLaunchKernelGGL((gated_group_norm_kernel<TG, TO>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream,
+                           (TO*)out, out_stride, o, w, (const TG*)gate, gate_stride, eps, rows, N, group, scale);
+      });
+    });
+    if (rc | inner) return 1;
+    HIP_LAUNCH_CHECK();
+    return 0;
+  }
+  if (scale == 1.0f && out_stride == N && gate_dt != DT_F32 && gate_dt == out_dt && N % 8 == 0 && gate_stride % 8 == 0 && aligned16(gate) && aligned16(o) &&
       aligned16(w) && aligned16(out)) {
     const int rv = by_dtype(gate_dt, [&](auto* tg) {
       using TG = std::remove_pointer_t<decltype(tg)>;
@@ -528,8 +584,8 @@ VDAMD_API int vdamd_gated_rms_norm(void* out, const float* o, const float* w, co
     using TG = std::remove_pointer_t<decltype(tg)>;
     inner = by_dtype(out_dt, [&](auto* to) {
       using TO = std::remove_pointer_t<decltype(to)>;
-      hipLaunchKernelGGL((gated_rms_norm_kernel<TG, TO>), dim3(rows), dim3(row_threads(N)), 0, stream, (TO*)out, o, w,
-                         (const TG*)gate, gate_stride, eps, N);
+      hipLaunchKernelGGL((gated_rms_norm_kernel<TG, TO>), dim3(rows), dim3(row_threads(N)), 0, stream, (TO*)out,
+                         out_stride, o, w, (const TG*)gate, gate_stride, eps, N, scale);
     });
   });
   if (rc | inner) return 1;
@@ -628,8 +684,8 @@ VDAMD_API int vdamd_decay_linear_attention(float* out, const void* x, long x_str
 VDAMD_API int vdamd_latent_prep(void* out, const void* q, long q_st, long q_sh, int nope, const void* q_lat, long l_sh,
                                 long l_st, const void* latent, long lat_st, const float* norm_w, float eps,
                                 const float* inv_freq, int half, float rs, const int* positions, void* cache,
-                                void* vfrag, const int* slot_mapping, int T, int H, int rank, int rope, int bs, int dt,
-                                hipStream_t stream) {
+                                void* vfrag, const int* slot_mapping, int T, int H, int rank, int rope, int bs,
+                                int interleaved, int dt, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || rank <= 0 || rope < 0 || 2 * half > rope) return 1;
   if (vfrag != nullptr && (latent == nullptr || rank % 16 || bs <= 0 || bs % 8)) return 1;
@@ -638,7 +694,7 @@ VDAMD_API int vdamd_latent_prep(void* out, const void* q, long q_st, long q_sh, 
     using TT = std::remove_pointer_t<decltype(tp)>;
     hipLaunchKernelGGL((latent_prep_kernel<TT>), dim3(T), dim3(256), 0, stream, (TT*)out, (const TT*)q, q_st, q_sh, nope,
                        (const TT*)q_lat, l_sh, l_st, (const TT*)latent, lat_st, norm_w, eps, inv_freq, half, rs,
-                       positions, (TT*)cache, (TT*)vfrag, slot_mapping, H, rank, rope, bs);
+                       positions, (TT*)cache, (TT*)vfrag, slot_mapping, H, rank, rope, bs, interleaved);
   });
   if (rc) return 1;
   HIP_LAUNCH_CHECK();
@@ -647,16 +703,18 @@ VDAMD_API int vdamd_latent_prep(void* out, const void* q, long q_st, long q_sh, 
 
 VDAMD_API int vdamd_latent_row_attention(void* out, const void* q, const void* cache, const int* block_table,
                                          long bt_stride, const int* token_seq, const int* seq_lens, float scale, int T,
-                                         int H, int dk, int rank, int bs, int dt, hipStream_t stream) {
+                                         int H, int dk, int rank, int bs, int window, const float* sinks,
+                                         const void* gate, long gate_stride, int dt, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (H <= 0 || rank <= 0 || rank > dk || dk > 4096 || rank > 1024 || bs <= 0) return 1;
+  if (H <= 0 || rank <= 0 || rank > dk || dk > 4096 || rank > 1024 || bs <= 0 || window < 0) return 1;
   const dim3 grid(T, (H + 3) / 4);
   const size_t lds = (size_t)4 * dk * sizeof(float);
   const int rc = by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
 #define LRA(NV_)                                                                                                      \
   hipLaunchKernelGGL((latent_row_attention_kernel<TT, NV_>), grid, dim3(256), lds, stream, (TT*)out, (const TT*)q,     \
-                     (const TT*)cache, block_table, bt_stride, token_seq, seq_lens, scale, H, dk, rank, bs)
+                     (const TT*)cache, block_table, bt_stride, token_seq, seq_lens, scale, H, dk, rank, bs, window,     \
+                     sinks, (const TT*)gate, gate_stride)
     if (rank <= 64) LRA(1);
     else if (rank <= 128) LRA(2);
     else if (rank <= 256) LRA(4);

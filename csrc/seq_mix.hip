@@ -7,10 +7,15 @@
 //   conv_norm_cache        causal per-channel convolution over time of a fused [q | k | v | ..] projection (history
 //                          from the chunk itself or from a per-request state slot), per-head RMS norm of q and k,
 //                          value mixing, k / v into row caches, q out
+//                          (the head norms are optional; with frequencies given, q and k heads are then rotated by
+//                          their position, value i paired with value i + half)
+//   short_conv_act         the convolution alone over the leading columns of a fused projection, through SiLU when
+//                          asked, result in the activation type
 //   conv_state_update      the last taps-1 projected rows of every sequence into its state slot
 //   window_bias_attention  attention over the caches K [blocks, Hkv, block, D] (key rows) and V [blocks, Hkv,
 //                          block / 8, Dv, 8] (8 keys side by side per channel: the V^T operand of the matrix cores
-//                          is one 16-byte load): causal window that keeps the first keys, score cap, logarithmic
+//                          is one 16-byte load): causal window that keeps the first keys (or blocks of `chunk`
+//                          positions counted from the sequence's start), score cap, logarithmic
 //                          distance bias, sink in the denominator, sigmoid gate on the output, online softmax in
 //                          fp32.  Two kernels: a matrix-core one for bf16 (16 query rows x 32 keys per wave and
 //                          step, softmax weights fed to the matrix cores as a high and a low bf16 part so that they
@@ -209,10 +214,19 @@ struct ConvArgs {
   const int* slot_mapping;                  // [T]
   int T, H, G, D, Dv, taps, block_size;
   float eps;
+  const float* inv_freq; int rot_half;      // [rot_half] fp32 or null: q and k heads rotated, pairs rot_half apart
 };
+
+__device__ __forceinline__ void conv_rotate(float u, float v, int pos, float freq, float& ou, float& ov) {
+  const float ang = (float)pos * freq;
+  const float cs = cosf(ang), sn = sinf(ang);
+  ou = u * cs - v * sn;
+  ov = v * cs + u * sn;
+}
 
 template <typename T>
 __global__ void conv_norm_cache_kernel(ConvArgs a) {
+  __shared__ float rot_lds[4][64 * UNIT_MAX_PER_LANE];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int s = a.token_seq ? a.token_seq[t] : t;
@@ -258,7 +272,7 @@ __global__ void conv_norm_cache_kernel(ConvArgs a) {
         ss += v * v;
       }
     }
-    if (kind < 2) {
+    if (kind < 2 && a.q_norm != nullptr) {
       ss = wave_sum(ss);
       const float inv = 1.0f / sqrtf(ss / (float)width + a.eps);
       const float* nw = kind == 0 ? a.q_norm : a.k_norm;
@@ -267,6 +281,26 @@ __global__ void conv_norm_cache_kernel(ConvArgs a) {
         const int cl = lane + it * 64;
         if (cl < width) acc[it] = acc[it] * inv * nw[cl];
       }
+    }
+    if (kind < 2 && a.rot_half > 0) {             // (uniform over the wave) partners meet through the wave's LDS row
+      float* rl = rot_lds[wave];
+#pragma unroll
+      for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+        const int cl = lane + it * 64;
+        if (cl < width) rl[cl] = acc[it];
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int it = 0; it < UNIT_MAX_PER_LANE; ++it) {
+        const int cl = lane + it * 64;
+        if (cl < 2 * a.rot_half) {
+          const int pi = cl < a.rot_half ? cl : cl - a.rot_half;
+          float ou, ov;
+          conv_rotate(rl[pi], rl[pi + a.rot_half], pos, a.inv_freq[pi], ou, ov);
+          acc[it] = cl < a.rot_half ? ou : ov;
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
     if (kind == 0) {
       T* q = (T*)a.q_out + ((long)t * a.H + head) * a.D;
@@ -362,7 +396,7 @@ __device__ __forceinline__ void conv_vec_token(const ConvArgs& a, int t, int tas
       for (int e = 0; e < 8; ++e) acc[e] += (float)wv[e] * (float)u[e];
     }
   }
-  if (kind < 2) {
+  if (kind < 2 && a.q_norm != nullptr) {
     float ss = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ss += acc[e] * acc[e];
@@ -373,6 +407,26 @@ __device__ __forceinline__ void conv_vec_token(const ConvArgs& a, int t, int tas
       const float* nw = (kind == 0 ? a.q_norm : a.k_norm) + 8 * li;
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = acc[e] * inv * nw[e];
+    }
+  }
+  if (a.rot_half > 0 && !is_v) {                   // (uniform over the wave; rot_half is a multiple of 8 here)
+    // a lane's 8 values lie wholly in the first half, the second half or the unrotated rest; the partner's 8 values
+    // are rot_half / 8 lanes up or down, inside the same unit
+    const int shift = a.rot_half >> 3;
+    const int region = 8 * li < a.rot_half ? 0 : (8 * li < 2 * a.rot_half ? 1 : 2);
+    const int src = region == 0 ? lane + shift : (region == 1 ? lane - shift : lane);
+    float other[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) other[e] = __shfl(acc[e], src & 63, 64);
+    if (region < 2) {
+      const int p0 = 8 * li - (region == 1 ? a.rot_half : 0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float ou, ov;
+        if (region == 0) conv_rotate(acc[e], other[e], pos, a.inv_freq[p0 + e], ou, ov);
+        else conv_rotate(other[e], acc[e], pos, a.inv_freq[p0 + e], ou, ov);
+        acc[e] = region == 0 ? ou : ov;
+      }
     }
   }
   if (!live) return;
@@ -446,6 +500,68 @@ __global__ void conv_state_update_kernel(const T* __restrict__ x, long x_stride,
   for (int k = 0; k < R; ++k) stf(st + (long)k * C + c, keep[k]);
 }
 
+// The convolution alone (no head structure): out[t, c] = act(sum_j w[j, c] * u[t - taps + 1 + j, c]) for the first C
+// columns of x, history from the step's own rows or the state slot as above.  One thread per (row, channel); the 16-bit
+// variant gives a thread 8 neighbouring channels (16-byte accesses).  A sequence's only row moves its state on here.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void short_conv_act_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ x,
+                                                             long x_stride, const T* __restrict__ w, T* __restrict__ state,
+                                                             const int* __restrict__ slots, const int* __restrict__ qsl,
+                                                             const int* __restrict__ seq_lens,
+                                                             const int* __restrict__ token_seq,
+                                                             const int* __restrict__ positions, int C, int taps, int silu) {
+  constexpr int W = VEC ? 8 : 1;
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * W;
+  if (c >= C) return;
+  const int s = token_seq ? token_seq[t] : t;
+  const int n = qsl[s + 1] - qsl[s];
+  const int pos = positions[t];
+  const int chunk_start = seq_lens[s] - n;
+  const int R = taps - 1;
+  T* st = state + (long)slots[s] * (R > 0 ? R : 1) * C;
+  const bool own_state = (n == 1) && R > 0;
+  float acc[W];
+#pragma unroll
+  for (int e = 0; e < W; ++e) acc[e] = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int back = taps - 1 - j;
+    const int p = pos - back;
+    if constexpr (VEC) {
+      using V8 = typename Vec8<T>::type;
+      const V8 wv = ld8<T>(w + (long)j * C + c);
+      V8 u;
+      if (p >= chunk_start && p >= 0) u = ld8<T>(x + (long)(t - back) * x_stride + c);
+      else if (p >= 0) u = ld8<T>(st + (long)(R - (chunk_start - p)) * C + c);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = (T)0.f;
+      }
+      if (own_state && j >= 1) st8<T>(st + (long)(j - 1) * C + c, u);       // (row j - 1 was read one turn earlier)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (float)wv[e] * (float)u[e];
+    } else {
+      float u = 0.f;
+      if (p >= chunk_start && p >= 0) u = ldf(x + (long)(t - back) * x_stride + c);
+      else if (p >= 0) u = ldf(st + (long)(R - (chunk_start - p)) * C + c);
+      if (own_state && j >= 1) stf(st + (long)(j - 1) * C + c, u);
+      acc[0] += ldf(w + (long)j * C + c) * u;
+    }
+  }
+  if (silu) {
+#pragma unroll
+    for (int e = 0; e < W; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
+  }
+  if constexpr (VEC) {
+    typename Vec8<T>::type o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (T)acc[e];
+    st8<T>(out + (long)t * out_stride + c, o);
+  } else {
+    stf(out + (long)t * out_stride + c, acc[0]);
+  }
+}
+
 // ------------------------------------------------------------------------------------------- attention
 struct AttnArgs {
   const void* q;                    // [T, H, D]
@@ -458,6 +574,7 @@ struct AttnArgs {
   void* out;                        // [T, H, Dv]
   int T, H, G, D, Dv, block_size, window, keep_first;
   float scale, softcap;
+  int chunk;                        // > 0: a query sees only the keys of its own block of `chunk` positions
 };
 
 template <typename T, bool VEC> struct RowDot;
@@ -512,8 +629,9 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
   const int pos = a.positions[t];
   const T* q = (const T*)a.q + ((long)t * a.H + h) * a.D;
   for (int d = lane; d < a.D; d += 64) sq[d] = ldf(q + d);
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int nkeep = a.window > 0 ? min(a.keep_first, lo) : 0;
+  int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  if (a.chunk > 0) lo = max(lo, pos - pos % a.chunk);
+  const int nkeep = a.window > 0 && a.chunk == 0 ? min(a.keep_first, lo) : 0;
   const int total = nkeep + (pos - lo + 1);
   const float r1 = a.bias_scale ? a.bias_scale[h] : 0.f, r2 = a.bias_rate ? a.bias_rate[h] : 0.f;
   const int* bt = a.block_table + (long)s * a.bt_stride;
@@ -649,8 +767,10 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   // ---- key steps of the wave: [0, kept) and [window start of its first row, position of its last row]
   const int p_first = start + min(tok0, max(n_tok - 1, 0));
   const int p_last = start + min(tok0 + tpw - 1, max(n_tok - 1, 0));
-  const int lo_min = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
-  const int nkeep = a.window > 0 ? min(a.keep_first, lo_min) : 0;
+  int lo_min = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  if (a.chunk > 0) lo_min = max(lo_min, p_first - p_first % a.chunk);
+  const int keep_first = a.chunk > 0 ? 0 : a.keep_first;
+  const int nkeep = a.window > 0 ? min(keep_first, lo_min) : 0;
   int start_b = lo_min & ~31;
   int n_a = (nkeep + 31) >> 5;
   if (start_b < (n_a << 5)) { start_b = 0; n_a = 0; }
@@ -669,10 +789,12 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
 #pragma unroll
   for (int c = 0; c < VT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  const int lo_row = a.window > 0 ? pos - a.window + 1 : 0;
+  int lo_row = a.window > 0 ? pos - a.window + 1 : 0;
+  if (a.chunk > 0) lo_row = max(lo_row, pos - pos % a.chunk);
   // a step all of whose 32 keys every row of the wave sees needs no mask: inside [window start of the wave's
   // last row, position of its first row], or inside the kept first keys
-  const int full_lo = a.window > 0 ? p_last - a.window + 1 : 0;
+  int full_lo = a.window > 0 ? p_last - a.window + 1 : 0;
+  if (a.chunk > 0) full_lo = max(full_lo, p_last - p_last % a.chunk);
   const float posf = (float)pos;
   const float cap_in = a.softcap > 0.f ? 2.f / a.softcap : 0.f, cap_out = a.softcap * LOG2E;
   // newest keys first: with a distance bias they carry the largest scores, so the running maximum settles in the
@@ -680,7 +802,7 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   for (int it = wk; it < n_steps; it += kw) {
     const int si = n_steps - 1 - it;
     const int base = si < n_a ? (si << 5) : start_b + ((si - n_a) << 5);
-    const bool interior = base + 31 <= p_first && (base >= full_lo || base + 31 < a.keep_first);
+    const bool interior = base + 31 <= p_first && (base >= full_lo || base + 31 < keep_first);
     // K rows of the two interleaved tiles
     const int key0 = base + 8 * (r16 >> 2) + (r16 & 3);
     const int ka = min(key0, p_last), kb = min(key0 + 4, p_last);
@@ -722,7 +844,7 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int key = kidx0 + j;
-        const bool seen = row_ok && key <= pos && (key >= lo_row || key < a.keep_first);
+        const bool seen = row_ok && key <= pos && (key >= lo_row || key < keep_first);
         p[j] = seen ? p[j] : -INFINITY;            // (also drops the NaN a negative distance gives the logarithm)
       }
     }
@@ -902,17 +1024,20 @@ VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* co
                                     const float* q_norm, const float* k_norm, const float* v_first,
                                     const float* v_lambda, float* v_keep, void* q_out, void* k_cache, void* v_cache,
                                     const int* slot_mapping, int T, int B, int H, int G, int D, int Dv, int taps,
-                                    int block_size, float eps, int update_multi, int dt, hipStream_t stream) {
+                                    int block_size, float eps, int update_multi, const float* inv_freq, int rot_half,
+                                    int dt, hipStream_t stream) {
   if (T <= 0) return 0;
   if (taps < 1 || taps > CONV_MAX_TAPS || D > 64 * UNIT_MAX_PER_LANE || Dv > 64 * UNIT_MAX_PER_LANE || H % G ||
-      block_size <= 0 || (v_first != nullptr && v_lambda == nullptr))
+      block_size <= 0 || (v_first != nullptr && v_lambda == nullptr) || (q_norm == nullptr) != (k_norm == nullptr) ||
+      rot_half < 0 || 2 * rot_half > D || (rot_half > 0 && inv_freq == nullptr))
     return 1;
   ConvArgs a{x, x_stride, conv_w, state, slots, qsl, seq_lens, token_seq, positions, q_norm, k_norm, v_first, v_lambda,
-             v_keep, q_out, k_cache, v_cache, slot_mapping, T, H, G, D, Dv, taps, block_size, eps};
+             v_keep, q_out, k_cache, v_cache, slot_mapping, T, H, G, D, Dv, taps, block_size, eps, inv_freq, rot_half};
   const int units = H + 2 * G;
   const int waves = units >= 4 ? 4 : units;
   const int C = H * D + G * (D + Dv), R = taps - 1;
-  const bool vec = dt != DT_F32 && D % 8 == 0 && Dv % 8 == 0 && D <= 512 && Dv <= 512 && x_stride % 8 == 0;
+  const bool vec = dt != DT_F32 && D % 8 == 0 && Dv % 8 == 0 && D <= 512 && Dv <= 512 && x_stride % 8 == 0 &&
+                   rot_half % 8 == 0;
   auto pack = [](int width, int& gs, int& upw) {        // lanes per unit, units per wave
     gs = width / 8;
     upw = (gs & (gs - 1)) == 0 ? 64 / gs : 1;
@@ -933,6 +1058,38 @@ VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* co
     }
     if (!vec || std::is_same_v<TT, float>)
       hipLaunchKernelGGL((conv_norm_cache_kernel<TT>), dim3(T), dim3(64 * waves), 0, stream, a);
+    if (update_multi && R > 0)
+      hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3((C + 255) / 256, B), dim3(256), 0, stream,
+                         (const TT*)x, x_stride, (TT*)state, slots, qsl, C, R);
+  });
+}
+
+// out [T, out_stride] = act(conv over time of x[:, :C]); state [slots, max(taps - 1, 1), C] moves on.  update_multi: 0
+// when every sequence of the step has one row
+VDAMD_API int vdamd_short_conv_act(void* out, long out_stride, const void* x, long x_stride, const void* conv_w,
+                                   void* state, const int* slots, const int* qsl, const int* seq_lens,
+                                   const int* token_seq, const int* positions, int T, int B, int C, int taps, int silu,
+                                   int update_multi, int dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (taps < 1 || taps > CONV_MAX_TAPS || C <= 0) return 1;
+  const int R = taps - 1;
+  const bool vec = dt != DT_F32 && C % 8 == 0 && x_stride % 8 == 0 && out_stride % 8 == 0 &&
+                   ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0;
+  return by_dtype(dt, [&](auto* tp) {
+    using TT = std::remove_pointer_t<decltype(tp)>;
+    bool done = false;
+    if constexpr (!std::is_same_v<TT, float>) {
+      if (vec) {
+        hipLaunchKernelGGL((short_conv_act_kernel<TT, true>), dim3(T, (C / 8 + 255) / 256), dim3(256), 0, stream,
+                           (TT*)out, out_stride, (const TT*)x, x_stride, (const TT*)conv_w, (TT*)state, slots, qsl,
+                           seq_lens, token_seq, positions, C, taps, silu);
+        done = true;
+      }
+    }
+    if (!done)
+      hipLaunchKernelGGL((short_conv_act_kernel<TT, false>), dim3(T, (C + 255) / 256), dim3(256), 0, stream, (TT*)out,
+                         out_stride, (const TT*)x, x_stride, (const TT*)conv_w, (TT*)state, slots, qsl, seq_lens,
+                         token_seq, positions, C, taps, silu);
     if (update_multi && R > 0)
       hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3((C + 255) / 256, B), dim3(256), 0, stream,
                          (const TT*)x, x_stride, (TT*)state, slots, qsl, C, R);
@@ -966,14 +1123,14 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
                                           const float* bias_scale, const float* bias_rate, const float* sinks,
                                           const void* gate, long gate_stride, void* out, int T, int B, int H, int G,
                                           int D, int Dv, int block_size, int window, int keep_first,
-                                          int max_query_len, float scale, float softcap, int use_mfma, int dt,
-                                          hipStream_t stream) {
+                                          int max_query_len, float scale, float softcap, int use_mfma, int chunk,
+                                          int dt, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H % G || D <= 0 || Dv <= 0 || Dv > 64 * ATTN_V_PER_LANE || block_size <= 0 || block_size % 8 ||
-      (bias_scale && !bias_rate))
+      (bias_scale && !bias_rate) || chunk < 0)
     return 1;
   AttnArgs a{q, k_cache, v_cache, block_table, bt_stride, token_seq, positions, bias_scale, bias_rate, sinks, gate,
-             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap};
+             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap, chunk};
   const int qpg = H / G;
   const int dtiles = D / 32, vtiles = Dv / 16;
   if (use_mfma && dt == DT_BF16 && qsl && seq_lens && B > 0 && max_query_len > 0 && D % 32 == 0 && Dv % 16 == 0 &&

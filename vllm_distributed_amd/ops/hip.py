@@ -68,17 +68,24 @@ def load() -> ctypes.CDLL:
         "vdamd_scalar_norm": [P, P, P, F, I, I, L, I, I, P],
         "vdamd_scalar_norm_residual": [P, P, P, P, P, F, I, I, L, I, I, P],
         "vdamd_poly_norm": [P, P, P, F, I, I, L, I, P],
-        "vdamd_conv_norm_cache": [P, L] + [P] * 16 + [I] * 8 + [F, I, I, P],
-        "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, P, P, L, P] + [I] * 10 + [F, F, I, I, P],
+        "vdamd_conv_norm_cache": [P, L] + [P] * 16 + [I] * 8 + [F, I, P, I, I, P],
+        "vdamd_short_conv_act": [P, L, P, L, P, P, P, P, P, P, P] + [I] * 7 + [P],
+        "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, P, P, L, P] + [I] * 10 + [F, F, I, I, I, P],
+        "vdamd_residual_rms": [P, L, P, L, P, L, P, L, P, L, P, P, F, F, I, I, I, I, I, I, P],
+        "vdamd_gelu_mul_rows": [P, P, L, P, L, P, I, I, I, I, I, P],
+        "vdamd_sigmoid_mul": [P, L, P, L, P, L, F, I, I, I, P],
+        "vdamd_gelu": [P, P, L, I, I, P],
+        "vdamd_delta_rule_prep": [P, P, P, P, P, L, P, L, P, L, P, P, I, I, I, I, F, I, P],
+        "vdamd_gated_delta_rule": [P, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
         "vdamd_embed_scaled": [P, P, P, F, I, I, I, I, P],
         "vdamd_layer_norm_to": [P, P, L, P, L, P, P, F, I, I, I, I, I, P],
-        "vdamd_gated_rms_norm": [P, P, P, P, L, F, I, I, I, I, P],
+        "vdamd_gated_rms_norm": [P, L, P, P, P, L, F, I, I, I, F, I, I, P],
         "vdamd_clamped_glu": [P, P, L, I, I, F, F, I, P],
         "vdamd_relu_squared": [P, P, L, I, P],
         "vdamd_expert_epilogue": [P, P, P, L, P, P, I, I, P, P, L, I, I, I, P],
         "vdamd_decay_linear_attention": [P, P, L, P, P, P, P, P, I, I, I, I, I, I, I, P],
-        "vdamd_latent_prep": [P, P, L, L, I, P, L, L, P, L, P, F, P, I, F, P, P, P, P, I, I, I, I, I, I, P],
-        "vdamd_latent_row_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, P],
+        "vdamd_latent_prep": [P, P, L, L, I, P, L, L, P, L, P, F, P, I, F, P, P, P, P, I, I, I, I, I, I, I, P],
+        "vdamd_latent_row_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, P, P, L, I, P],
     }
     for name, argtypes in sigs.items():
         fn = getattr(lib, name)
@@ -1293,7 +1300,7 @@ WINDOW_ATTENTION_MFMA = os.environ.get("VDAMD_WINDOW_ATTENTION_MFMA", "1") != "0
 
 def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions, num_heads: int,
                     num_kv_heads: int, dim: int, vdim: int, q_norm, k_norm, eps: float, v_first, v_lambda,
-                    keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True):
+                    keep_v: bool, k_cache, v_cache, slot_mapping, has_prefill: bool = True, inv_freq=None):
     t = x.shape[0]
     c = num_heads * dim + num_kv_heads * (dim + vdim)
     taps = conv_weight.shape[0]
@@ -1321,21 +1328,24 @@ def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, tok
         assert v_first.shape == (t, gv) and v_first.dtype == torch.float32 and v_first.is_contiguous()
     q = torch.empty((t, num_heads, dim), dtype=x.dtype, device=x.device)
     kept = torch.empty((t, gv), dtype=torch.float32, device=x.device) if keep_v else None
+    half = 0 if inv_freq is None else int(inv_freq.numel())
+    assert 2 * half <= dim and (q_norm is None) == (k_norm is None)
     _check(_LIB.vdamd_conv_norm_cache(
         x.data_ptr(), x.stride(0), conv_weight.data_ptr(), state.data_ptr(), _i32(slots, "slots").data_ptr(),
         _i32(query_start_loc, "query_start_loc").data_ptr(), _i32(seq_lens, "seq_lens").data_ptr(),
         _ptr(_i32(token_seq, "token_seq")), _i32(positions, "positions").data_ptr(),
-        _f32_vec(q_norm, dim, "q_norm").data_ptr(), _f32_vec(k_norm, dim, "k_norm").data_ptr(),
+        _ptr(_f32_vec(q_norm, dim, "q_norm")), _ptr(_f32_vec(k_norm, dim, "k_norm")),
         _ptr(v_first), _ptr(_f32_vec(v_lambda, 1, "v_lambda")) if v_first is not None else None, _ptr(kept),
         q.data_ptr(), _ptr(k_cache), _ptr(v_cache), _i32(slot_mapping, "slot_mapping").data_ptr(),
-        t, b, num_heads, num_kv_heads, dim, vdim, taps, bs, float(eps), 1 if has_prefill else 0, _dt(x), _stream()),
+        t, b, num_heads, num_kv_heads, dim, vdim, taps, bs, float(eps), 1 if has_prefill else 0,
+        _ptr(_f32_vec(inv_freq, half, "inv_freq")) if half else None, half, _dt(x), _stream()),
         "conv_norm_cache")
     return q, kept
 
 
 def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
                           scale: float, softcap: float, window: int, keep_first: int, bias_scale, bias_rate, sinks,
-                          gate, max_query_len: int = 0, out=None):
+                          gate, max_query_len: int = 0, out=None, chunk: int = 0):
     t, h, d = q.shape
     g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     b = seq_lens.shape[0]
@@ -1360,7 +1370,7 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
         _ptr(_f32_vec(bias_scale, h, "bias_scale")), _ptr(_f32_vec(bias_rate, h, "bias_rate")),
         _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride, out.data_ptr(), t, b, h, g, d, dv, bs,
         int(window), int(keep_first), int(max_query_len) if max_query_len else t, float(scale), float(softcap),
-        1 if WINDOW_ATTENTION_MFMA else 0, _dt(q), _stream()), "window_bias_attention")
+        1 if WINDOW_ATTENTION_MFMA else 0, int(chunk), _dt(q), _stream()), "window_bias_attention")
     return out
 
 
@@ -1423,13 +1433,18 @@ def decay_linear_attention(x: torch.Tensor, num_heads: int, dim: int, vdim: int,
 
 
 def gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, eps: float,
-                   out_dtype: torch.dtype) -> torch.Tensor:
+                   out_dtype: torch.dtype, group: int = 0, scale: float = 1.0, out=None) -> torch.Tensor:
     t, n = o.shape
     assert o.dtype == torch.float32 and o.is_contiguous() and gate.shape == (t, n) and gate.stride(1) == 1
-    out = torch.empty((t, n), dtype=out_dtype, device=o.device)
-    _check(_LIB.vdamd_gated_rms_norm(out.data_ptr(), o.data_ptr(), _f32_vec(weight, n, "weight").data_ptr(),
-                                     gate.data_ptr(), gate.stride(0), float(eps), t, n, _dt(gate), _DT[out_dtype],
-                                     _stream()), "gated_rms_norm")
+    group = int(group or 0)
+    assert group == 0 or n % group == 0
+    if out is None:
+        out = torch.empty((t, n), dtype=out_dtype, device=o.device)
+    assert out.dim() == 2 and out.shape == (t, n) and out.stride(1) == 1
+    _check(_LIB.vdamd_gated_rms_norm(out.data_ptr(), out.stride(0), o.data_ptr(),
+                                     _f32_vec(weight, group or n, "weight").data_ptr(), gate.data_ptr(), gate.stride(0),
+                                     float(eps), t, n, group, float(scale), _dt(gate), _dt(out), _stream()),
+           "gated_rms_norm")
     return out
 
 
@@ -1454,7 +1469,7 @@ def relu_squared(x: torch.Tensor) -> torch.Tensor:
 def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optional[torch.Tensor],
                 norm_weight: Optional[torch.Tensor], eps: float, inv_freq: torch.Tensor, rot_scale: float,
                 positions: torch.Tensor, cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
-                fragments: Optional[torch.Tensor] = None) -> torch.Tensor:
+                fragments: Optional[torch.Tensor] = None, interleaved: bool = False) -> torch.Tensor:
     """``fragments``: the V^T fragment cache ``[blocks, 1, rank / 16, block / 8, 16, 8]`` of the matrix-core latent
     attention kernel, written beside the rows when the layer keeps one."""
     t, h, qd = q.shape
@@ -1482,14 +1497,14 @@ def latent_prep(q: torch.Tensor, nope: int, q_lat: torch.Tensor, latent: Optiona
         q_lat.stride(1), latent.data_ptr() if write else None, latent.stride(0) if write else 0,
         _f32_vec(norm_weight, rank, "norm_weight").data_ptr() if write else None, float(eps), inv_freq.data_ptr(),
         half, float(rot_scale), positions.data_ptr(), cache.data_ptr() if write else None, _ptr(fragments),
-        slot_mapping.data_ptr() if write else None, t, h, rank, rope, cache.shape[2] if write else 8, _dt(q),
-        _stream()), "latent_prep")
+        slot_mapping.data_ptr() if write else None, t, h, rank, rope, cache.shape[2] if write else 8,
+        1 if interleaved else 0, _dt(q), _stream()), "latent_prep")
     return out
 
 
 def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
                          token_seq: Optional[torch.Tensor], seq_lens: torch.Tensor, scale: float, rank: int,
-                         max_seq_len: int = 0) -> torch.Tensor:
+                         max_seq_len: int = 0, window: int = 0, sinks=None, gate=None) -> torch.Tensor:
     t, h, dk = q.shape
     assert q.is_contiguous() and cache.is_contiguous() and cache.dtype == q.dtype
     assert cache.shape[1] == 1 and cache.shape[3] == dk and 0 < rank <= dk
@@ -1497,10 +1512,15 @@ def latent_row_attention(q: torch.Tensor, cache: torch.Tensor, block_table: torc
     assert seq_lens.numel() >= t and (token_seq is None or (token_seq.dtype == torch.int32 and token_seq.numel() >= t))
     assert token_seq is not None or block_table.shape[0] >= t
     out = torch.empty((t, h, rank), dtype=q.dtype, device=q.device)
+    gate_stride = 0
+    if gate is not None:
+        assert gate.dim() == 2 and gate.shape[0] >= t and gate.shape[1] == h and gate.stride(1) == 1 and gate.dtype == q.dtype
+        gate_stride = gate.stride(0)
     _check(_LIB.vdamd_latent_row_attention(out.data_ptr(), q.data_ptr(), cache.data_ptr(), block_table.data_ptr(),
                                            block_table.stride(0), None if token_seq is None else token_seq.data_ptr(),
-                                           seq_lens.data_ptr(), float(scale), t, h, dk, rank, cache.shape[2], _dt(q),
-                                           _stream()), "latent_row_attention")
+                                           seq_lens.data_ptr(), float(scale), t, h, dk, rank, cache.shape[2],
+                                           int(window), _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride,
+                                           _dt(q), _stream()), "latent_row_attention")
     return out
 
 
@@ -1522,4 +1542,133 @@ def expert_epilogue(routed: torch.Tensor, x: torch.Tensor, topw: Optional[torch.
                                       None if shared is None else gate.data_ptr(),
                                       0 if shared is None else gate.stride(0), t, h, _dt(routed), _stream()),
            "expert_epilogue")
+    return out
+
+
+
+# ------------------------------------------------ fp32 residual stream with RMS norms, side inputs per token,
+# ------------------------------------------------ convolution + activation, the gated delta rule
+def _rows2d(t: torch.Tensor, name: str) -> torch.Tensor:
+    assert t.dim() == 2 and t.stride(1) == 1 and t.is_cuda, f"{name}: rows of a 2-D tensor with unit column stride"
+    return t
+
+
+def _residual_rms(x, a, b, y, post_w, w, eps, out_dtype, offset, normed) -> torch.Tensor:
+    rows, h = _rows2d(x, "x").shape
+    adds = a is not None or y is not None
+    if adds:
+        assert x.dtype == torch.float32, "the residual stream is fp32"
+    in_dt = _dt(x)
+    for t, name in ((a, "a"), (b, "b"), (y, "y")):
+        if t is not None:
+            assert _rows2d(t, name).shape == (rows, h)
+            in_dt = _dt(t)
+    for u, v in ((a, b), (a, y), (b, y)):
+        assert u is None or v is None or u.dtype == v.dtype
+    assert b is None or a is not None
+    out = torch.empty((rows, h), dtype=out_dtype, device=x.device)
+    _check(_LIB.vdamd_residual_rms(
+        out.data_ptr(), h, x.data_ptr(), x.stride(0), _ptr(a), 0 if a is None else a.stride(0), _ptr(b),
+        0 if b is None else b.stride(0), _ptr(y), 0 if y is None else y.stride(0),
+        _ptr(_f32_vec(post_w, h, "post_weight")) if y is not None else None, _ptr(_f32_vec(w, h, "weight")),
+        float(offset), float(eps), rows, h, 1 if normed else 0, _dt(x), in_dt, _DT[out_dtype], _stream()), "residual_rms")
+    return out
+
+
+def rms_norm_to(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+                offset: float = 0.0) -> torch.Tensor:
+    lead = x.shape[:-1]
+    x2 = x if x.dim() == 2 else x.reshape(-1, x.shape[-1])
+    return _residual_rms(x2, None, None, None, None, weight, eps, out_dtype, offset, True).view(lead + (x.shape[-1],))
+
+
+def add_rms_norm_to(residual, a, b, weight, eps: float, out_dtype, offset: float = 0.0, normed: bool = True):
+    assert residual.is_contiguous()
+    return _residual_rms(residual, a, b, None, None, weight, eps, out_dtype, offset, normed)
+
+
+def norm_add_norm(y, post_weight, residual, next_weight, eps: float, out_dtype, next_offset: float = 0.0,
+                  next_normed: bool = True):
+    assert residual.is_contiguous()
+    return _residual_rms(residual, None, None, y, post_weight, next_weight, eps, out_dtype, next_offset, next_normed)
+
+
+def gelu_mul_rows(g: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col: int) -> torch.Tensor:
+    rows, n = _rows2d(g, "g").shape
+    assert _rows2d(table, "table").dtype == g.dtype and 0 <= col and col + n <= table.shape[1]
+    assert ids.dtype == torch.int32 and ids.numel() >= rows and ids.is_contiguous()
+    out = torch.empty((rows, n), dtype=g.dtype, device=g.device)
+    _check(_LIB.vdamd_gelu_mul_rows(out.data_ptr(), g.data_ptr(), g.stride(0), table.data_ptr(), table.stride(0),
+                                    ids.data_ptr(), int(col), n, rows, table.shape[0], _dt(g), _stream()), "gelu_mul_rows")
+    return out
+
+
+def sigmoid_mul(o: torch.Tensor, gate: torch.Tensor, scale: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    rows, n = _rows2d(o, "o").shape
+    assert _rows2d(gate, "gate").shape == (rows, n) and gate.dtype == o.dtype
+    if out is None:
+        out = torch.empty((rows, n), dtype=o.dtype, device=o.device)
+    assert _rows2d(out, "out").shape == (rows, n) and out.dtype == o.dtype
+    _check(_LIB.vdamd_sigmoid_mul(out.data_ptr(), out.stride(0), o.data_ptr(), o.stride(0), gate.data_ptr(),
+                                  gate.stride(0), float(scale), rows, n, _dt(o), _stream()), "sigmoid_mul")
+    return out
+
+
+def gelu(x: torch.Tensor, tanh: bool) -> torch.Tensor:
+    xc = x if x.is_contiguous() else x.contiguous()
+    out = torch.empty_like(xc)
+    _check(_LIB.vdamd_gelu(out.data_ptr(), xc.data_ptr(), xc.numel(), 1 if tanh else 0, _dt(xc), _stream()), "gelu")
+    return out
+
+
+def short_conv_act(x, channels: int, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions,
+                   silu: bool, has_prefill: bool = True) -> torch.Tensor:
+    t = _rows2d(x, "x").shape[0]
+    c, taps = int(channels), conv_weight.shape[0]
+    r = max(taps - 1, 1)
+    b = seq_lens.shape[0]
+    assert x.shape[1] >= c and conv_weight.shape == (taps, c) and conv_weight.dtype == x.dtype and conv_weight.is_contiguous()
+    assert 1 <= taps <= CONV_MAX_TAPS
+    assert state is not None and state.dtype == x.dtype and state.is_contiguous() and state.shape[1:] == (r, c), \
+        (None if state is None else state.shape, (r, c))
+    assert slots.shape[0] == b and query_start_loc.shape[0] >= b + 1 and positions.shape[0] >= t
+    assert token_seq is None or token_seq.shape[0] >= t
+    assert token_seq is not None or t <= b, "rows without a sequence"
+    assert int(state.shape[0]) > 0
+    out = torch.empty((t, c), dtype=x.dtype, device=x.device)
+    _check(_LIB.vdamd_short_conv_act(
+        out.data_ptr(), c, x.data_ptr(), x.stride(0), conv_weight.data_ptr(), state.data_ptr(),
+        _i32(slots, "slots").data_ptr(), _i32(query_start_loc, "query_start_loc").data_ptr(),
+        _i32(seq_lens, "seq_lens").data_ptr(), _ptr(_i32(token_seq, "token_seq")),
+        _i32(positions, "positions").data_ptr(), t, b, c, taps, 1 if silu else 0, 1 if has_prefill else 0, _dt(x),
+        _stream()), "short_conv_act")
+    return out
+
+
+def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, beta, dt, dt_bias, a_log, state, slots,
+                     query_start_loc, seq_lens, norm_eps: float = 1e-6, max_query_len: int = 0) -> torch.Tensor:
+    t = _rows2d(x, "x").shape[0]
+    h, g = int(num_heads), int(num_qk_heads)
+    b = seq_lens.shape[0]
+    assert h % g == 0 and 0 < dim <= 256 and x.shape[1] >= 2 * g * dim + h * vdim
+    assert _rows2d(beta, "beta").shape[0] >= t and beta.shape[1] == h and beta.dtype == x.dtype
+    assert _rows2d(dt, "dt").shape[0] >= t and dt.shape[1] == h * dim and dt.dtype == x.dtype
+    assert state is not None and state.dtype == torch.float32 and state.is_contiguous()
+    assert tuple(state.shape[1:]) == (h, dim, vdim), (tuple(state.shape), (h, dim, vdim))
+    assert slots.shape[0] == b and query_start_loc.shape[0] >= b + 1
+    dev = x.device
+    qn = torch.empty((t, g, dim), dtype=torch.float32, device=dev)
+    kn = torch.empty((t, g, dim), dtype=torch.float32, device=dev)
+    decay = torch.empty((t, h, dim), dtype=torch.float32, device=dev)
+    bsig = torch.empty((t, h), dtype=torch.float32, device=dev)
+    out = torch.empty((t, h * vdim), dtype=torch.float32, device=dev)
+    _check(_LIB.vdamd_delta_rule_prep(
+        qn.data_ptr(), kn.data_ptr(), decay.data_ptr(), bsig.data_ptr(), x.data_ptr(), x.stride(0), beta.data_ptr(),
+        beta.stride(0), dt.data_ptr(), dt.stride(0), _f32_vec(dt_bias, h * dim, "dt_bias").data_ptr(),
+        _f32_vec(a_log, h, "a_log").data_ptr(), t, h, g, dim, float(norm_eps), _dt(x), _stream()), "delta_rule_prep")
+    _check(_LIB.vdamd_gated_delta_rule(
+        out.data_ptr(), x.data_ptr(), x.stride(0), 2 * g * dim, qn.data_ptr(), kn.data_ptr(), decay.data_ptr(),
+        bsig.data_ptr(), state.data_ptr(), _i32(slots, "slots").data_ptr(),
+        _i32(query_start_loc, "query_start_loc").data_ptr(), _i32(seq_lens, "seq_lens").data_ptr(), b, h, g, dim, vdim,
+        _dt(x), _stream()), "gated_delta_rule")
     return out
