@@ -139,10 +139,10 @@ def _parse():
     ap.add_argument("--alt-parallelism", type=str, default="pp",
                     help="second layout measured in a child process after the headline when N > 1 ('none' = skip)")
     ap.add_argument("--alt-timeout", type=float, default=900.0)
-    ap.add_argument("--family-compare", type=str, default=None, choices=[None, "tavulix", "kabapel"],
+    ap.add_argument("--family-compare", type=str, default=None, choices=[None, "tavulix", "kabapel", "gosizen"],
                     help="instead of the headline: prefill and decode throughput of this model family at a few layer "
                          "sizes beside the closest existing family at equal size (Tavulix: Gemma-2; Kabapel: "
-                         "DeepSeek-V2), random weights, one GPU")
+                         "DeepSeek-V2; Gosizen: Kabapel), random weights, one GPU")
     ap.add_argument("--compare-sizes", type=str, default="small,medium",
                     help="with --family-compare: which of small / medium / large to run")
     ap.add_argument("--compare-only", type=str, default=None,
@@ -274,6 +274,31 @@ def _kabapel_models(z: dict) -> dict:
     return {"kabapel": ("kabapel-tiny", kab), "deepseek_v2": ("deepseek-v2-lite", dsk)}
 
 
+def _gosizen_models(z: dict) -> dict:
+    """The same layer sizes as a Gosizen config (parallel and latent layers in turn, every layer with an expert block
+    and a token side input) and as a Kabapel config (recurrent and latent layers in turn around an fp32 residual
+    stream, expert blocks: the closest family the framework has)."""
+    vocab = 32000
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]}, "router": {"experts": z["experts"] + z["identity"], "top": z["top"]}}
+    window = min(z["prompt"], 1024)
+    lat = {"heads": z["heads"], "dim": z["nope"], "rot_dim": z["rope"], "vdim": z["vdim"], "kv_rank": z["rank"],
+           "q_rank": max(z["width"] // 2, 64), "scale": (z["nope"] + z["rope"]) ** -0.5, "mask": {"size": window},
+           "rot": {"base": 10000.0, "dims": z["rope"]}}
+    kv = max(z["heads"] // 4, 1)
+    par = {"left": {"heads": z["heads"], "kv_heads": kv, "dim": z["nope"], "vdim": z["vdim"], "conv": 4,
+                    "scale": z["nope"] ** -0.5, "mask": {"size": window},
+                    "rot": {"base": 10000.0, "dims": z["nope"],
+                            "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 4096}}},
+           "right": {"heads": z["heads"], "kv_heads": z["heads"], "dim": z["nope"], "vdim": z["vdim"], "conv": 4,
+                     "decay_rank": 64, "gate_rank": 64},
+           "left_scale": 0.5, "right_scale": 0.5}
+    layers = [{"type": "parallel" if i % 2 == 0 else "latent_attention", "mixer": par if i % 2 == 0 else lat, "mlp": moe}
+              for i in range(z["layers"])]
+    gos = {"architecture": "Gosizen", "vocab": vocab, "width": z["width"], "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+           "token_side": {"dim": 64}, "layers": layers}
+    return {"gosizen": ("gosizen-tiny", gos), "kabapel": _kabapel_models(z)["kabapel"]}
+
+
 def run_family_compare(args) -> None:
     """Prefill throughput (``prompts`` prompts of ``prompt`` tokens, one generated token each) and decode
     throughput (``batch`` sequences, 64 further tokens each; the prefill time measured the same way is taken off)
@@ -283,10 +308,12 @@ def run_family_compare(args) -> None:
     from vllm_distributed_amd import LLM, SamplingParams
     os.environ.setdefault("VLLM_LOGGING_LEVEL", "WARNING")
     rows = []
-    kabapel = args.family_compare == "kabapel"
+    kabapel = args.family_compare in ("kabapel", "gosizen")
     for size in [s for s in args.compare_sizes.split(",") if s]:
         z = (KABAPEL_SIZES if kabapel else COMPARE_SIZES)[size]
-        for family, (base, over) in (_kabapel_models(z) if kabapel else _compare_models(z)).items():
+        models = (_gosizen_models(z) if args.family_compare == "gosizen" else _kabapel_models(z)) if kabapel \
+            else _compare_models(z)
+        for family, (base, over) in models.items():
             if args.compare_only and family != args.compare_only:
                 continue
             llm = LLM(model=base, hf_overrides=over, dtype=args.dtype, device=args.device, load_format="dummy",

@@ -4,13 +4,13 @@
 //   delta_rule_prep   per row: q and k of every query / key head made unit vectors (q times dim^-0.5), the decays
 //                     g = exp(-exp(a_log[h]) * softplus(dt + dt_bias)) per head and key channel, b = sigmoid(beta);
 //                     all fp32, computed once per row instead of once per lane of the recurrence
-//   gated_delta_rule  per (sequence, head, tile of value columns) one wave walks the sequence's rows:
+//   gated_delta_rule  per (sequence, head, tile of 64 value columns) a workgroup walks the sequence's rows:
 //                       S <- g * S (by rows) ; u = b (v - S^T k) ; S <- S + k u^T ; o = S^T q
 //                     as ONE read of the decayed state per row - r = (gS)^T k and p = (gS)^T q together, then
-//                     u = b (v - r), o = p + (k.q) u, S = gS + k u^T.  The wave's 64 lanes are CT columns x RP row parts;
-//                     a lane keeps R = ceil(dim / RP) rows of one column in registers, the row parts are summed with
-//                     xor-shuffles (no LDS, no barrier), and the next row's q / k / g are loaded while the current one
-//                     is computed.  A prompt portion and a single decoded row are the same kernel.
+//                     u = b (v - r), o = p + (k.q) u, S = gS + k u^T.  A lane keeps a quarter of one column of S in
+//                     registers; the quarters are summed with two xor-shuffles; q / k / g / v / b of a chunk of rows
+//                     are staged in LDS with the next chunk's loads in flight (one barrier per chunk).  A prompt
+//                     portion and a single decoded row are the same kernel.
 #include "common.h"
 #include <math.h>
 #include <type_traits>
@@ -63,32 +63,41 @@ __global__ __launch_bounds__(256) void delta_rule_prep_kernel(float* __restrict_
   for (int h = threadIdx.x; h < H; h += blockDim.x) bsig[t * H + h] = 1.0f / (1.0f + expf(-ldf(beta + t * beta_stride + h)));
 }
 
-template <int RP> __device__ __forceinline__ float parts_sum(float v) {
-  // lanes are (row part) * CT + column: sum over the row parts
-#pragma unroll
-  for (int o = 64 / RP; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+// sum over the four row parts of a wave (lanes are part * 16 + column)
+__device__ __forceinline__ float parts_sum(float v) {
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
   return v;
 }
 
-// grid (column tiles, H, sequences), one wave.  x rows hold [.. | v (H * vdim)] at column v_off; qn / kn [T, G, dim],
-// decay [T, H, dim], bsig [T, H] fp32; out [T, H * vdim] fp32; state [slots, H, dim, vdim] fp32.
-template <typename T, int R, int RP>
-__global__ __launch_bounds__(64) void gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ x,
-                                                              long x_stride, int v_off, const float* __restrict__ qn,
-                                                              const float* __restrict__ kn,
-                                                              const float* __restrict__ decay,
-                                                              const float* __restrict__ bsig, float* __restrict__ state,
-                                                              const int* __restrict__ slots, const int* __restrict__ qsl,
-                                                              const int* __restrict__ seq_lens, int H, int G, int dim,
-                                                              int vdim) {
-  constexpr int CT = 64 / RP;
-  const int lane = threadIdx.x;
-  const int col = blockIdx.x * CT + (lane & (CT - 1));
-  const int part = lane / CT;
+// grid (tiles of 64 value columns, H, sequences), 4 waves: wave w owns columns 16 w .. 16 w + 15 of the tile, a lane
+// (part = lane / 16, column = lane % 16) keeps rows part * R .. part * R + R - 1 of its column of S in registers
+// (4 R >= dim).  The sequence's rows are walked in chunks of C: q, k, g (all of the head, fp32), v (the tile's columns)
+// and b of a chunk are staged in LDS by the whole workgroup - the next chunk's loads are in flight while the current
+// one is computed, one barrier per chunk - and read back as broadcasts (16-byte reads: a lane's rows are neighbours).
+// x rows hold v (H * vdim) at column v_off; qn / kn [T, G, dim], decay [T, H, dim], bsig [T, H] fp32; out
+// [T, H * vdim] fp32; state [slots, H, dim, vdim] fp32.
+template <typename T, int R, int C>
+__global__ __launch_bounds__(256) void gated_delta_rule_kernel(float* __restrict__ out, const T* __restrict__ x,
+                                                               long x_stride, int v_off, const float* __restrict__ qn,
+                                                               const float* __restrict__ kn,
+                                                               const float* __restrict__ decay,
+                                                               const float* __restrict__ bsig, float* __restrict__ state,
+                                                               const int* __restrict__ slots, const int* __restrict__ qsl,
+                                                               const int* __restrict__ seq_lens, int H, int G, int dim,
+                                                               int vdim) {
+  constexpr int DP = 4 * R;                         // rows, padded (rows past dim stay zero)
+  constexpr int ROW = 3 * DP + 64 + 4;              // floats staged per sequence row: q | k | g | v (64) | b, pad
+  constexpr int NST = (C * ROW + 255) / 256;        // staged values per thread and chunk
+  __shared__ __attribute__((aligned(16))) float lds[2][C * ROW];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int cl = lane & 15, part = lane >> 4;
+  const int col0 = blockIdx.x * 64;
+  const int col = col0 + wave * 16 + cl;
   const int h = blockIdx.y, s = blockIdx.z;
   const int g = h / (H / G);
   const int q0 = qsl[s], n = qsl[s + 1] - q0;
-  if (n <= 0) return;
+  if (n <= 0) return;                               // (the whole workgroup)
   const bool col_ok = col < vdim;
   const int ccol = col_ok ? col : vdim - 1;
   const int r0 = part * R;
@@ -97,44 +106,69 @@ __global__ __launch_bounds__(64) void gated_delta_rule_kernel(float* __restrict_
   const bool fresh = seq_lens[s] - n <= 0;          // the rows start the sequence: whatever the slot holds is not ours
 #pragma unroll
   for (int i = 0; i < R; ++i) S[i] = (!fresh && r0 + i < dim) ? st[(long)(r0 + i) * vdim] : 0.f;
-  float qc[R], kc[R], gc[R], qx[R], kx[R], gx[R];
-  float vc, bc, vx = 0.f, bx = 0.f;
-  auto load = [&](long t, float* q, float* k, float* gg, float& v, float& b) {
-    const float* qp = qn + (t * G + g) * (long)dim + r0;
-    const float* kp = kn + (t * G + g) * (long)dim + r0;
-    const float* gp = decay + (t * H + h) * (long)dim + r0;
+
+  float stage[NST];
+  auto fetch = [&](int chunk) {                     // this thread's share of a chunk, global -> registers
+    const int rows = min(C, n - chunk * C);
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      const bool ok = r0 + i < dim;
-      q[i] = ok ? qp[i] : 0.f;
-      k[i] = ok ? kp[i] : 0.f;
-      gg[i] = ok ? gp[i] : 0.f;
+    for (int e = 0; e < NST; ++e) {
+      const int idx = tid + e * 256;
+      const int j = idx / ROW, f = idx - j * ROW;
+      float val = 0.f;
+      if (j < rows) {
+        const long t = q0 + chunk * C + j;
+        if (f < DP) { if (f < dim) val = qn[(t * G + g) * (long)dim + f]; }
+        else if (f < 2 * DP) { if (f - DP < dim) val = kn[(t * G + g) * (long)dim + f - DP]; }
+        else if (f < 3 * DP) { if (f - 2 * DP < dim) val = decay[(t * H + h) * (long)dim + f - 2 * DP]; }
+        else if (f < 3 * DP + 64) { if (col0 + f - 3 * DP < vdim) val = ldf(x + t * x_stride + v_off + (long)h * vdim + col0 + f - 3 * DP); }
+        else if (f == 3 * DP + 64) val = bsig[t * H + h];
+      }
+      stage[e] = val;
     }
-    v = ldf(x + t * x_stride + v_off + (long)h * vdim + ccol);
-    b = bsig[t * H + h];
   };
-  load(q0, qc, kc, gc, vc, bc);
-  for (int i = 0; i < n; ++i) {
-    const long t = q0 + i;
-    if (i + 1 < n) load(t + 1, qx, kx, gx, vx, bx);
-    float r = 0.f, p = 0.f, kq = 0.f;
+  auto stash = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < R; ++j) {
-      S[j] *= gc[j];
-      r += S[j] * kc[j];
-      p += S[j] * qc[j];
-      kq += kc[j] * qc[j];
+    for (int e = 0; e < NST; ++e) {
+      const int idx = tid + e * 256;
+      if (idx < C * ROW) lds[buf][idx] = stage[e];
     }
-    r = parts_sum<RP>(r);
-    p = parts_sum<RP>(p);
-    kq = parts_sum<RP>(kq);
-    const float u = bc * (vc - r);
+  };
+  const int chunks = (n + C - 1) / C;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int c = 0; c < chunks; ++c) {
+    if (c + 1 < chunks) fetch(c + 1);
+    const float* base = lds[c & 1];
+    const int rows = min(C, n - c * C);
+    for (int j = 0; j < rows; ++j) {
+      const float* L = base + j * ROW;
+      float r = 0.f, p = 0.f, kq = 0.f;
+      float kr[R];
 #pragma unroll
-    for (int j = 0; j < R; ++j) S[j] += kc[j] * u;
-    if (part == 0 && col_ok) out[t * (long)H * vdim + (long)h * vdim + col] = p + kq * u;
+      for (int i = 0; i < R; i += 4) {
+        const f32x4 qv = *reinterpret_cast<const f32x4*>(L + r0 + i);
+        const f32x4 kv = *reinterpret_cast<const f32x4*>(L + DP + r0 + i);
+        const f32x4 gv = *reinterpret_cast<const f32x4*>(L + 2 * DP + r0 + i);
 #pragma unroll
-    for (int j = 0; j < R; ++j) { qc[j] = qx[j]; kc[j] = kx[j]; gc[j] = gx[j]; }
-    vc = vx; bc = bx;
+        for (int e = 0; e < 4; ++e) {
+          S[i + e] *= gv[e];
+          r += S[i + e] * kv[e];
+          p += S[i + e] * qv[e];
+          kq += kv[e] * qv[e];
+          kr[i + e] = kv[e];
+        }
+      }
+      r = parts_sum(r);
+      p = parts_sum(p);
+      kq = parts_sum(kq);
+      const float u = L[3 * DP + 64] * (L[3 * DP + wave * 16 + cl] - r);
+#pragma unroll
+      for (int i = 0; i < R; ++i) S[i] += kr[i] * u;
+      if (part == 0 && col_ok) out[(long)(q0 + c * C + j) * H * vdim + (long)h * vdim + col] = p + kq * u;
+    }
+    if (c + 1 < chunks) stash((c + 1) & 1);
+    __syncthreads();
   }
   if (col_ok) {
 #pragma unroll
@@ -169,19 +203,17 @@ VDAMD_API int vdamd_gated_delta_rule(float* out, const void* x, long x_stride, i
                                      int vdim, int dtype, hipStream_t stream) {
   if (B <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || dim <= 0 || dim > 256 || vdim <= 0) return 1;
-  // row parts so that a lane keeps at most 16 rows; fewer parts (more columns per wave) for small heads
-  const int rp = dim <= 64 ? 4 : (dim <= 128 ? 8 : 16);
-  const int ct = 64 / rp;
-  const int r = (dim + rp - 1) / rp;
-  const dim3 grid((vdim + ct - 1) / ct, H, B);
+  const int r = (dim + 3) / 4;                      // rows per lane
+  const dim3 grid((vdim + 63) / 64, H, B);
   const int rc = by_dtype(dtype, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
-#define GDR(R_, RP_)                                                                                                 \
-  hipLaunchKernelGGL((gated_delta_rule_kernel<TT, R_, RP_>), grid, dim3(64), 0, stream, out, (const TT*)x, x_stride,   \
+#define GDR(R_, C_)                                                                                                  \
+  hipLaunchKernelGGL((gated_delta_rule_kernel<TT, R_, C_>), grid, dim3(256), 0, stream, out, (const TT*)x, x_stride,   \
                      v_off, qn, kn, decay, bsig, state, slots, qsl, seq_lens, H, G, dim, vdim)
-    if (rp == 4) { if (r <= 4) GDR(4, 4); else if (r <= 8) GDR(8, 4); else GDR(16, 4); }
-    else if (rp == 8) { if (r <= 12) GDR(12, 8); else GDR(16, 8); }
-    else { if (r <= 12) GDR(12, 16); else GDR(16, 16); }
+    if (r <= 8) GDR(8, 8);
+    else if (r <= 16) GDR(16, 8);
+    else if (r <= 32) GDR(32, 8);
+    else GDR(64, 4);
 #undef GDR
   });
   if (rc) return 1;

@@ -92,6 +92,21 @@ __device__ __forceinline__ void mla_st(void* cache, long off, float v) {
   }
 }
 
+// What a layer may add to plain causal attention: a sliding window (a token sees its last `window` keys; 0 = all), a
+// learned sink per head whose exponential joins the softmax denominator, a sigmoid gate per (token, head) on the output.
+struct MlaExtra {
+  int window;
+  const float* sinks;                // [Hq] or null
+  const void* gate; long gate_stride;  // [T, gate_stride] raw values of the element type, or null
+};
+
+// l (relative to the running maximum m, log2 scale) and the factor the accumulators take when the sink joins
+__device__ __forceinline__ void mla_add_sink(float sink_log2, float m, float& l, float& factor) {
+  const float m_f = fmaxf(m, sink_log2);
+  factor = fast_exp2(m - m_f);
+  l = l * factor + fast_exp2(sink_log2 - m_f);
+}
+
 // P2: the fp32 softmax weights enter the PV product as a high and a low 16-bit part (two MFMAs per tile, ~16
 // mantissa bits) instead of being rounded to 8 bits: for models that define their attention weights in 32-bit.
 template <typename T, int DK, int DV, bool KV8, bool P2>
@@ -99,7 +114,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     T* __restrict__ out, long out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const T* __restrict__ q, long q_stride, const void* __restrict__ k_cache, const void* __restrict__ v_cache,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ token_seq,
-    const int* __restrict__ seq_lens, float scale_log2e, int Hq, int block_size, int num_splits) {
+    const int* __restrict__ seq_lens, float scale_log2e, int Hq, int block_size, int num_splits, MlaExtra ex) {
   using V = typename Vec8<T>::type;
   constexpr int KSTEPS = DK / 32;              // 32-wide steps of the QK^T reduction
   constexpr int KS = (KSTEPS + 3) / 4;         // ... per wave (the last waves may run short: zero Q there)
@@ -115,10 +130,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int seq_len = seq_lens[t];
   const int* bt_row = block_table + (long)(token_seq != nullptr ? token_seq[t] : t) * bt_stride;
 
-  const int n_groups = (seq_len + 31) >> 5;
+  // keys [win_lo, seq_len): nothing in front of win_lo is read (its pages may have gone back to the pool)
+  const int win_lo = ex.window > 0 ? max(seq_len - ex.window, 0) : 0;
+  const int g_lo = win_lo >> 5;
+  const int n_groups = ((seq_len + 31) >> 5) - g_lo;
   const int gps = (n_groups + num_splits - 1) / num_splits;
-  const int g_begin = split * gps;
-  const int g_end = min(g_begin + gps, n_groups);
+  const int g_begin = g_lo + split * gps;
+  const int g_end = min(g_begin + gps, g_lo + n_groups);
 
   // this wave's k-steps: global step wid * KS + s, clamped for the address and zeroed in Q when past the end
   V qf[KS];
@@ -144,7 +162,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int base = g * 32;
     // K rows of the two interleaved S^T tiles: tile 0 row i <-> key 8 (i >> 2) + (i & 3), tile 1 the same + 4
     const int key0 = base + 8 * (r16 >> 2) + (r16 & 3);
-    const int ka = min(key0, seq_len - 1), kb = min(key0 + 4, seq_len - 1);
+    const int ka = max(min(key0, seq_len - 1), win_lo), kb = max(min(key0 + 4, seq_len - 1), win_lo);
     const long ra = ((long)bt_row[ka / block_size] * block_size + (ka % block_size)) * DK;
     const long rb = ((long)bt_row[kb / block_size] * block_size + (kb % block_size)) * DK;
 #pragma unroll
@@ -153,7 +171,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       f.kb[s] = mla_ld<T, KV8>(k_cache, rb + kstep_off[s]);
     }
     // V^T: this lane's 8 keys are base + 8 g4 .. + 7 (inside one block: block_size % 8 == 0)
-    const int vkey = min(base + 8 * g4, seq_len - 1) & ~7;
+    const int vkey = max(min(base + 8 * g4, seq_len - 1), win_lo) & ~7;
     const long vo = (long)bt_row[vkey / block_size] * (DV / 16) * slab + ((vkey % block_size) >> 3) * 128 + 8 * r16;
 #pragma unroll
     for (int i = 0; i < VT; ++i) f.vf[i] = mla_ld<T, KV8>(v_cache, vo + (long)(wid * VT + i) * slab);
@@ -189,7 +207,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float sv = (j < 4 ? s0[j & 3] : s1[j & 3]) * scale_log2e;
-      p[j] = (kidx0 + j < seq_len) ? sv : MLA_NEG_BIG;
+      p[j] = (kidx0 + j < seq_len && kidx0 + j >= win_lo) ? sv : MLA_NEG_BIG;
       tmax = fmaxf(tmax, p[j]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
@@ -224,7 +242,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (r16 >= nq) return;
   const int qh = qh0 + r16;
   if (num_splits == 1) {
-    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+    float factor = 1.f;
+    if (ex.sinks != nullptr) mla_add_sink(ex.sinks[qh] * 1.4426950408889634f, m, lsum, factor);
+    float inv = lsum > 0.f ? factor / lsum : 0.f;
+    if (ex.gate != nullptr) inv *= 1.f / (1.f + __expf(-(float)((const T*)ex.gate)[t * ex.gate_stride + qh]));
     T* orow = out + t * out_stride + (long)qh * DV + 4 * g4;
 #pragma unroll
     for (int i = 0; i < VT; ++i) {
@@ -257,7 +278,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     T* __restrict__ out, long out_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
     const T* __restrict__ q, long q_stride, const void* __restrict__ k_cache, const void* __restrict__ v_cache,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ token_seq,
-    const int* __restrict__ seq_lens, float scale_log2e, int T_, int Hq, int block_size, int num_splits) {
+    const int* __restrict__ seq_lens, float scale_log2e, int T_, int Hq, int block_size, int num_splits,
+    MlaExtra ex) {
   using V = typename Vec8<T>::type;
   constexpr int KSTEPS = DK / 32;
   constexpr int KS = (KSTEPS + 3) / 4;
@@ -305,10 +327,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int n = 0; n < NQ; ++n) seq_len = max(seq_len, slen[n]);
   const int* bt_row = block_table + (long)seq_row * bt_stride;
 
-  const int n_groups = (seq_len + 31) >> 5;
+  // every tile's own window start; nothing in front of the earliest one is read
+  int wlo[NQ];
+  int win_lo = seq_len;
+#pragma unroll
+  for (int n = 0; n < NQ; ++n) {
+    wlo[n] = ex.window > 0 ? max(slen[n] - ex.window, 0) : 0;
+    if (slen[n] > 0) win_lo = min(win_lo, wlo[n]);
+  }
+  const int g_lo = win_lo >> 5;
+  const int n_groups = ((seq_len + 31) >> 5) - g_lo;
   const int gps = (n_groups + num_splits - 1) / num_splits;
-  const int g_begin = split * gps;
-  const int g_end = min(g_begin + gps, n_groups);
+  const int g_begin = g_lo + split * gps;
+  const int g_end = min(g_begin + gps, g_lo + n_groups);
 
   V qf[NQ][KS];
   int kstep_off[KS];
@@ -340,7 +371,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   auto load = [&](Frag& f, int g) {
     const int base = g * 32;
     const int key0 = base + 8 * (r16 >> 2) + (r16 & 3);
-    const int ka = min(key0, seq_len - 1), kb = min(key0 + 4, seq_len - 1);
+    const int ka = max(min(key0, seq_len - 1), win_lo), kb = max(min(key0 + 4, seq_len - 1), win_lo);
     const long ra = ((long)bt_row[ka / block_size] * block_size + (ka % block_size)) * DK;
     const long rb = ((long)bt_row[kb / block_size] * block_size + (kb % block_size)) * DK;
 #pragma unroll
@@ -348,7 +379,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       f.ka[s] = mla_ld<T, KV8>(k_cache, ra + kstep_off[s]);
       f.kb[s] = mla_ld<T, KV8>(k_cache, rb + kstep_off[s]);
     }
-    const int vkey = min(base + 8 * g4, seq_len - 1) & ~7;
+    const int vkey = max(min(base + 8 * g4, seq_len - 1), win_lo) & ~7;
     const long vo = (long)bt_row[vkey / block_size] * (DV / 16) * slab + ((vkey % block_size) >> 3) * 128 + 8 * r16;
 #pragma unroll
     for (int i = 0; i < VT; ++i) f.vf[i] = mla_ld<T, KV8>(v_cache, vo + (long)(wid * VT + i) * slab);
@@ -393,7 +424,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float sv = (j < 4 ? s0[j & 3] : s1[j & 3]) * scale_log2e;
-        p[j] = (kidx0 + j < slen[n]) ? sv : MLA_NEG_BIG;
+        p[j] = (kidx0 + j < slen[n] && kidx0 + j >= wlo[n]) ? sv : MLA_NEG_BIG;
         tmax = fmaxf(tmax, p[j]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
@@ -430,7 +461,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int qh = qh0[n] + r16;
     if (slen[n] <= 0 || qh >= Hq) continue;
     if (num_splits == 1) {
-      const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+      float factor = 1.f;
+      if (ex.sinks != nullptr) mla_add_sink(ex.sinks[qh] * 1.4426950408889634f, m[n], lsum, factor);
+      float inv = lsum > 0.f ? factor / lsum : 0.f;
+      if (ex.gate != nullptr) inv *= 1.f / (1.f + __expf(-(float)((const T*)ex.gate)[tok[n] * ex.gate_stride + qh]));
       T* orow = out + tok[n] * out_stride + (long)qh * DV + 4 * g4;
 #pragma unroll
       for (int i = 0; i < VT; ++i) {
@@ -452,14 +486,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 // Merge of the KV splits: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
 template <typename T, int DV>
 __global__ void mla_reduce_kernel(T* __restrict__ out, long out_stride, const float* __restrict__ part_o,
-                                  const float* __restrict__ part_ml, int Hq, int num_splits) {
+                                  const float* __restrict__ part_ml, int Hq, int num_splits, MlaExtra ex) {
   const int t = blockIdx.y, qh = blockIdx.x;
   const long p0 = ((long)t * Hq + qh) * num_splits;
   float mm = MLA_NEG_BIG;
   for (int s = 0; s < num_splits; ++s) mm = fmaxf(mm, part_ml[2 * (p0 + s)]);
-  float lt = 0.f;
+  const float sink2 = ex.sinks != nullptr ? ex.sinks[qh] * 1.4426950408889634f : MLA_NEG_BIG;
+  mm = fmaxf(mm, sink2);
+  float lt = ex.sinks != nullptr ? fast_exp2(sink2 - mm) : 0.f;
   for (int s = 0; s < num_splits; ++s) lt += part_ml[2 * (p0 + s) + 1] * fast_exp2(part_ml[2 * (p0 + s)] - mm);
-  const float inv = lt > 0.f ? 1.f / lt : 0.f;
+  float inv = lt > 0.f ? 1.f / lt : 0.f;
+  if (ex.gate != nullptr) inv *= 1.f / (1.f + __expf(-(float)((const T*)ex.gate)[t * ex.gate_stride + qh]));
   for (int d = threadIdx.x; d < DV; d += blockDim.x) {
     float o = 0.f;
     for (int s = 0; s < num_splits; ++s) o += part_o[(p0 + s) * DV + d] * fast_exp2(part_ml[2 * (p0 + s)] - mm);
@@ -544,7 +581,7 @@ template <typename T, int DK, int DV, bool KV8, bool P2>
 int launch_mla(void* out, long out_stride, void* part_o, void* part_ml, const void* q, long q_stride,
                const void* k_cache, const void* v_cache, const int* block_table, int bt_stride, const int* token_seq,
                const int* seq_lens, float scale, int T_, int Hq, int block_size, int num_splits, int mode,
-               hipStream_t st) {
+               MlaExtra ex, hipStream_t st) {
   const int q_tiles = (Hq + 15) / 16;
   const float sl2 = scale * 1.4426950408889634f;
   constexpr int NQ = 4;
@@ -552,20 +589,20 @@ int launch_mla(void* out, long out_stride, void* part_o, void* part_ml, const vo
     // (ids walk the tokens residue class by residue class: (T_ + NQ - 1) / NQ ids per class)
     mla_attention_multi_kernel<T, DK, DV, NQ, true, KV8, P2><<<dim3(num_splits, q_tiles, (T_ + NQ - 1) / NQ * NQ), 256, 0, st>>>(
         (T*)out, out_stride, (float*)part_o, (float*)part_ml, (const T*)q, q_stride, k_cache, v_cache, block_table,
-        bt_stride, token_seq, seq_lens, sl2, T_, Hq, block_size, num_splits);
+        bt_stride, token_seq, seq_lens, sl2, T_, Hq, block_size, num_splits, ex);
   } else if (mode == 2) {                           // NQ head tiles of a token share it
     mla_attention_multi_kernel<T, DK, DV, NQ, false, KV8, P2><<<dim3(num_splits, (q_tiles + NQ - 1) / NQ, T_), 256, 0, st>>>(
         (T*)out, out_stride, (float*)part_o, (float*)part_ml, (const T*)q, q_stride, k_cache, v_cache, block_table,
-        bt_stride, token_seq, seq_lens, sl2, T_, Hq, block_size, num_splits);
+        bt_stride, token_seq, seq_lens, sl2, T_, Hq, block_size, num_splits, ex);
   } else {
     mla_attention_kernel<T, DK, DV, KV8, P2><<<dim3(num_splits, q_tiles, T_), 256, 0, st>>>(
         (T*)out, out_stride, (float*)part_o, (float*)part_ml, (const T*)q, q_stride, k_cache, v_cache, block_table,
-        bt_stride, token_seq, seq_lens, sl2, Hq, block_size, num_splits);
+        bt_stride, token_seq, seq_lens, sl2, Hq, block_size, num_splits, ex);
   }
   HIP_LAUNCH_CHECK();
   if (num_splits > 1) {
     mla_reduce_kernel<T, DV><<<dim3(Hq, T_), 128, 0, st>>>((T*)out, out_stride, (const float*)part_o,
-                                                          (const float*)part_ml, Hq, num_splits);
+                                                          (const float*)part_ml, Hq, num_splits, ex);
     HIP_LAUNCH_CHECK();
   }
   return 0;
@@ -575,21 +612,21 @@ template <typename T>
 int dispatch_mla(int DK, int DV, int kv_fp8, void* out, long out_stride, void* part_o, void* part_ml, const void* q,
                  long q_stride, const void* k_cache, const void* v_cache, const int* block_table, int bt_stride,
                  const int* token_seq, const int* seq_lens, float scale, int T_, int Hq, int block_size,
-                 int num_splits, int mode, int precise, hipStream_t st) {
+                 int num_splits, int mode, int precise, MlaExtra ex, hipStream_t st) {
   if (precise && kv_fp8) return -6;       // (split weights over an 8-bit cache: not built)
 #define MLA_CASE(DK_, DV_)                                                                                        \
   if (DK == DK_ && DV == DV_) {                                                                                   \
     if (kv_fp8)                                                                                                   \
       return launch_mla<T, DK_, DV_, true, false>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache, \
                                                   block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq,     \
-                                                  block_size, num_splits, mode, st);                              \
+                                                  block_size, num_splits, mode, ex, st);                          \
     if (precise)                                                                                                  \
       return launch_mla<T, DK_, DV_, false, true>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache, \
                                                   block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq,     \
-                                                  block_size, num_splits, mode, st);                              \
+                                                  block_size, num_splits, mode, ex, st);                          \
     return launch_mla<T, DK_, DV_, false, false>(out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache, \
                                                  block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq,      \
-                                                 block_size, num_splits, mode, st);                               \
+                                                 block_size, num_splits, mode, ex, st);                           \
   }
   MLA_CASE(576, 512) MLA_CASE(96, 64) MLA_CASE(320, 256)
 #undef MLA_CASE
@@ -608,8 +645,11 @@ VDAMD_API int vdamd_mla_attention(void* out, long out_stride, void* part_o, void
                                   long q_stride, const void* k_cache, const void* v_cache, const int* block_table,
                                   int bt_stride, const int* token_seq, const int* seq_lens, float scale, int T_,
                                   int Hq, int DK, int DV, int block_size, int num_splits, int mode, int dtype,
-                                  int kv_fp8, int precise, void* stream) {
+                                  int kv_fp8, int precise, int window, const float* sinks, const void* gate,
+                                  long gate_stride, void* stream) {
   if (T_ <= 0) return 0;
+  if (window < 0) return -1;
+  const MlaExtra ex{window, sinks, gate, gate_stride};
   if (block_size % 8 || num_splits < 1 || num_splits > MLA_MAX_SPLITS) return -1;
   if (num_splits > 1 && (part_o == nullptr || part_ml == nullptr)) return -2;
   if (q_stride % 8 || out_stride % 4) return -5;
@@ -617,11 +657,11 @@ VDAMD_API int vdamd_mla_attention(void* out, long out_stride, void* part_o, void
   if (dtype == DT_BF16)
     return dispatch_mla<bf16_t>(DK, DV, kv_fp8, out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache,
                                 block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq, block_size, num_splits,
-                                mode, precise, st);
+                                mode, precise, ex, st);
   if (dtype == DT_F16)
     return dispatch_mla<f16_t>(DK, DV, kv_fp8, out, out_stride, part_o, part_ml, q, q_stride, k_cache, v_cache,
                                block_table, bt_stride, token_seq, seq_lens, scale, T_, Hq, block_size, num_splits,
-                               mode, precise, st);
+                               mode, precise, ex, st);
   return -3;
 }
 

@@ -278,8 +278,8 @@ class RowLatentAttention(Attention):
         # where the matrix-core latent kernel is built for this width and type, the values are cached once more as
         # its V^T fragments and it serves the layer (with fp32-precise softmax weights); else the plain kernel
         on_gpu = torch.empty(0).device.type != "cpu"       # (modules are built under the target device)
-        self.fragments = bool(on_gpu and dtype is not None and rank % 16 == 0 and not self.window
-                              and self.sink is None and ops.mla_kernel_ok(rank + rope, rank, dtype))
+        self.fragments = bool(on_gpu and dtype is not None and rank % 16 == 0
+                              and ops.mla_kernel_ok(rank + rope, rank, dtype))
         if source is not None:
             self.fragments = source.fragments
         if source is not None and (source.rank, source.rope) != (rank, rope):
@@ -323,7 +323,7 @@ class RowLatentAttention(Attention):
         if self.fragments:
             owner = self.source if self.source is not None else self
             return ops.mla_attention(qf, owner.k_cache, owner.v_cache, md.block_table, rows, lens, self.scale,
-                                     md.max_seq_len, precise=True)
+                                     md.max_seq_len, precise=True, window=self.window, sinks=self.sink, gate=gate)
         return ops.latent_row_attention(qf, self.rows, md.block_table, rows, lens, self.scale, self.rank, md.max_seq_len,
                                         self.window, self.sink, gate)
 

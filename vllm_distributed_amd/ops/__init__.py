@@ -600,13 +600,18 @@ def mla_cache_write(latent, k_cache, v_cache, slot_mapping):
 
 
 def mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out=None,
-                  precise: bool = False):
-    """``precise``: softmax weights with fp32 precision in the weighted sum (models that define them in 32-bit)."""
+                  precise: bool = False, window: int = 0, sinks=None, gate=None):
+    """``precise``: softmax weights with fp32 precision in the weighted sum (models that define them in 32-bit).
+    ``window`` / ``sinks`` / ``gate``: a sliding window, a sink per head in the denominator, a sigmoid gate per
+    (token, head) on the output (the matrix-core kernels only)."""
     on_hip = _use_hip(q) and _hip.mla_supported(q.shape[2], v_cache.shape[2] * v_cache.shape[4], q.dtype)
     _note_attention(q, on_hip)
     if on_hip:
         return _hip.mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out,
-                                  precise=precise)
+                                  precise=precise, window=window, sinks=sinks, gate=gate)
+    if window or sinks is not None or gate is not None:
+        raise NotImplementedError("window, sinks and gate exist in the matrix-core latent kernels only: layers that "
+                                  "use them elsewhere go through latent_row_attention")
     return torch_ref.mla_attention(q, k_cache, v_cache, block_table, token_seq, seq_lens, scale, max_seq_len, out)
 
 
