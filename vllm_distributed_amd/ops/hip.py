@@ -76,7 +76,7 @@ def load() -> ctypes.CDLL:
         "vdamd_sigmoid_mul": [P, L, P, L, P, L, F, I, I, I, P],
         "vdamd_gelu": [P, P, L, I, I, P],
         "vdamd_delta_rule_prep": [P, P, P, P, P, L, P, L, P, L, P, P, I, I, I, I, F, I, P],
-        "vdamd_gated_delta_rule": [P, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+        "vdamd_gated_delta_rule": [P, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "vdamd_embed_scaled": [P, P, P, F, I, I, I, I, P],
         "vdamd_layer_norm_to": [P, P, L, P, L, P, P, F, I, I, I, I, I, P],
         "vdamd_gated_rms_norm": [P, L, P, P, P, L, F, I, I, I, F, I, I, P],
@@ -1655,7 +1655,9 @@ def short_conv_act(x, channels: int, conv_weight, state, slots, query_start_loc,
 
 
 def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, beta, dt, dt_bias, a_log, state, slots,
-                     query_start_loc, seq_lens, norm_eps: float = 1e-6, max_query_len: int = 0) -> torch.Tensor:
+                     query_start_loc, seq_lens, norm_eps: float = 1e-6, max_query_len: int = 0,
+                     parts: int = 0) -> torch.Tensor:
+    """``max_query_len`` (0: unknown) only helps the kernel choose its tiling; ``parts`` forces one (benchmarks)."""
     t = _rows2d(x, "x").shape[0]
     h, g = int(num_heads), int(num_qk_heads)
     b = seq_lens.shape[0]
@@ -1669,7 +1671,7 @@ def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, 
     qn = torch.empty((t, g, dim), dtype=torch.float32, device=dev)
     kn = torch.empty((t, g, dim), dtype=torch.float32, device=dev)
     decay = torch.empty((t, h, dim), dtype=torch.float32, device=dev)
-    bsig = torch.empty((t, h), dtype=torch.float32, device=dev)
+    bsig = torch.empty((t, 2, h), dtype=torch.float32, device=dev)   # sigmoid(beta) | k.q of the head's group
     out = torch.empty((t, h * vdim), dtype=torch.float32, device=dev)
     _check(_LIB.vdamd_delta_rule_prep(
         qn.data_ptr(), kn.data_ptr(), decay.data_ptr(), bsig.data_ptr(), x.data_ptr(), x.stride(0), beta.data_ptr(),
@@ -1679,5 +1681,5 @@ def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, 
         out.data_ptr(), x.data_ptr(), x.stride(0), 2 * g * dim, qn.data_ptr(), kn.data_ptr(), decay.data_ptr(),
         bsig.data_ptr(), state.data_ptr(), _i32(slots, "slots").data_ptr(),
         _i32(query_start_loc, "query_start_loc").data_ptr(), _i32(seq_lens, "seq_lens").data_ptr(), b, h, g, dim, vdim,
-        _dt(x), _stream()), "gated_delta_rule")
+        int(max_query_len), int(parts), _dt(x), _stream()), "gated_delta_rule")
     return out
