@@ -1,8 +1,12 @@
 """Time the gated-delta-rule kernel (every tiling) beside the decayed linear attention kernel at equal head sizes:
 prompt portions and decode-only launches.  ``python benchmarks/delta_rule_bench.py`` on a GPU box; prints one table."""
-import torch
+import os
+import sys
 
-from vllm_distributed_amd.ops import hip
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+import torch  # noqa: E402
+
+from vllm_distributed_amd.ops import hip  # noqa: E402
 
 
 def timed(fn, reps=20):

@@ -123,6 +123,41 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(TO* __restrict__ 
   for (int i = lane; i < group; i += 64) stf(dst + i, orow[i] * inv * w[i] * sigmoid_f(ldf(g + i)) * scale);
 }
 
+// the same for 16-bit gate and result and runs of 8 L values, L a power of two up to 64: L neighbouring lanes per run, 8
+// values per lane in 16-byte accesses, the sum of squares over the L lanes by xor-shuffles (every lane takes part: the
+// lanes past the last run repeat it and store nothing)
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_norm_vec_kernel(T* __restrict__ out, long out_stride,
+                                                                   const float* __restrict__ o,
+                                                                   const float* __restrict__ w,
+                                                                   const T* __restrict__ gate, long gate_stride,
+                                                                   float eps, long units, int N, int group, int L,
+                                                                   float scale) {
+  using V8 = typename Vec8<T>::type;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const long unit = idx / L;
+  const int l = (int)(idx - unit * L);
+  const bool ok = unit < units;
+  const long u = ok ? unit : units - 1;
+  const int per_row = N / group;
+  const long row = u / per_row;
+  const int c0 = (int)(u - row * per_row) * group + 8 * l;
+  const float4* o4 = reinterpret_cast<const float4*>(o + row * (long)N + c0);
+  const float4 a = o4[0], b = o4[1];
+  float ss = a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+  for (int off = 1; off < L; off <<= 1) ss += __shfl_xor(ss, off, 64);
+  const float inv = 1.0f / sqrtf(ss / (float)group + eps) * scale;
+  const float4* w4 = reinterpret_cast<const float4*>(w + 8 * l);
+  const float4 wa = w4[0], wb = w4[1];
+  const V8 gv = ld8<T>(gate + row * gate_stride + c0);
+  const float of[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  const float wf[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+  V8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (T)(of[e] * inv * wf[e] * sigmoid_f((float)gv[e]));
+  if (ok) st8<T>(out + row * out_stride + c0, r);
+}
+
 // 16-bit gate and result, rows whose length and gate stride are multiples of 8: 16-byte accesses
 template <typename T>
 __global__ void gated_rms_norm_vec_kernel(T* __restrict__ out, const float* __restrict__ o, const float* __restrict__ w,
@@ -556,6 +591,20 @@ VDAMD_API int vdamd_gated_rms_norm(void* out, long out_stride, const float* o, c
   int inner = 0;
   if (group > 0) {
     const long units = (long)rows * (N / group);
+    const int L = group / 8;
+    if (gate_dt != DT_F32 && gate_dt == out_dt && group % 8 == 0 && L <= 64 && (L & (L - 1)) == 0 && out_stride % 8 == 0 &&
+        gate_stride % 8 == 0 && aligned16(gate) && aligned16(o) && aligned16(w) && aligned16(out)) {
+      const int rv = by_dtype(gate_dt, [&](auto* tg) {
+        using TG = std::remove_pointer_t<decltype(tg)>;
+        if constexpr (!std::is_same_v<TG, float>)
+          hipLaunchKernelGGL((gated_group_norm_vec_kernel<TG>), dim3((unsigned)((units * L + 255) / 256)), dim3(256), 0,
+                             stream, (TG*)out, out_stride, o, w, (const TG*)gate, gate_stride, eps, units, N, group, L,
+                             scale);
+      });
+      if (rv) return 1;
+      HIP_LAUNCH_CHECK();
+      return 0;
+    }
     const int rc = by_dtype(gate_dt, [&](auto* tg) {
       using TG = std::remove_pointer_t<decltype(tg)>;
       inner = by_dtype(out_dt, [&](auto* to) {

@@ -54,7 +54,7 @@ def test_residual_norms(dtype, h):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("n", [5, 16, 136])
+@pytest.mark.parametrize("n", [5, 16, 64, 128, 136])
 def test_gates_and_activations(dtype, n):
     hip = _hip()
     g = torch.Generator(device="cuda").manual_seed(n)
@@ -157,6 +157,34 @@ def test_chunked_attention(dtype, heads, kv, dim, vdim):
     table = torch.tensor([[3, 7, 1, 9, 0, 0], [2, 5, 8, 11, 4, 0], [6, 10, 0, 0, 0, 0]], dtype=torch.int32, device="cuda")
     sinks = torch.tensor([0.5, -1.0, 2.0, 0.0][:heads], device="cuda")
     for lens, rows in (([60, 80, 21], [1, 1, 1]), ([59, 70, 20], [45, 3, 20])):
+        t = sum(rows)
+        q = torch.randn(t, heads, dim, device="cuda", generator=g).to(dtype)
+        qsl = _i32(*[sum(rows[:i]) for i in range(4)])
+        seq = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, n in enumerate(rows)]).cuda()
+        pos = torch.cat([torch.arange(l - n, l, dtype=torch.int32) for l, n in zip(lens, rows)]).cuda()
+        decode = max(rows) == 1
+        got = hip.window_bias_attention(q, kc, vc, table, qsl, _i32(*lens), None if decode else seq, pos, dim ** -0.5, 0.0,
+                                        chunk, 0, None, None, sinks, None, max(rows), None, chunk)
+        want = torch_ref.window_bias_attention(q, kc, vc, table, qsl, _i32(*lens), dim ** -0.5, 0.0, chunk, 0, None, None,
+                                               sinks, None, chunk)
+        _close(got, want, dtype, 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("heads,kv,dim,vdim", [(2, 1, 128, 128), (4, 2, 64, 64), (2, 2, 40, 24)])
+def test_chunked_attention_over_many_pages(dtype, heads, kv, dim, vdim):
+    """Chunks of 150 positions over shuffled pages of 16 and sequences of several chunks: prompt portions that start
+    inside a chunk and cross one or two borders (whole key steps in front of a chunk's start are skipped), decoded rows
+    at a chunk's last and first position and deep inside the third chunk."""
+    hip = _hip()
+    g = torch.Generator(device="cuda").manual_seed(dim + 1)
+    bs, chunk, per = 16, 150, 27
+    nblk = 3 * per + 1
+    kc = (torch.randn(nblk, kv, bs, dim, device="cuda", generator=g) * 0.4).to(dtype)
+    vc = torch.randn(nblk, kv, bs // 8, vdim, 8, device="cuda", generator=g).to(dtype)
+    table = (torch.randperm(nblk - 1, device="cuda", generator=g) + 1).to(torch.int32).view(3, per)
+    sinks = torch.tensor([0.5, -1.0, 2.0, 0.0][:heads], device="cuda")
+    for lens, rows in (([300, 301, 425], [1, 1, 1]), ([340, 151, 430], [200, 3, 137]), ([150, 432, 17], [150, 300, 17])):
         t = sum(rows)
         q = torch.randn(t, heads, dim, device="cuda", generator=g).to(dtype)
         qsl = _i32(*[sum(rows[:i]) for i in range(4)])
