@@ -5,7 +5,7 @@
 //                     g = exp(-exp(a_log[h]) * softplus(dt + dt_bias)) per head and key channel, b = sigmoid(beta),
 //                     k.q of the unit vectors;
 //                     all fp32, computed once per row instead of once per lane of the recurrence
-//   gated_delta_rule  per (sequence, head, tile of 64 value columns) a workgroup walks the sequence's rows:
+//   gated_delta_rule  per (sequence, head, tile of 16 to 64 value columns) a workgroup walks the sequence's rows:
 //                       S <- g * S (by rows) ; u = b (v - S^T k) ; S <- S + k u^T ; o = S^T q
 //                     as ONE read of the decayed state per row - r = (gS)^T k and p = (gS)^T q together, then
 //                     u = b (v - r), o = p + (k.q) u, S = gS + k u^T.  A lane keeps a part (a 4th, 8th or 16th) of one

@@ -218,6 +218,18 @@ __global__ void embedding_kernel(T* __restrict__ out, const int* __restrict__ id
   for (int i = threadIdx.x; i < (H >> 3); i += blockDim.x) st8<T>(dst + 8 * i, ok ? ld8<T>(src + 8 * i) : zero);
 }
 
+// the same element by element, for rows that are not a whole number of 16-byte pieces
+template <typename T>
+__global__ void embedding_scalar_kernel(T* __restrict__ out, const int* __restrict__ ids, const T* __restrict__ w,
+                                        int H, int vocab_start, int rows) {
+  const long t = blockIdx.x;
+  const int id = ids[t] - vocab_start;
+  const bool ok = id >= 0 && id < rows;
+  const T* src = w + (long)(ok ? id : 0) * H;
+  T* dst = out + t * (long)H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ok ? src[i] : (T)0.f;
+}
+
 inline int norm_threads(int H) {
   int t = ((H >> 3) + NORM_MAX_ITERS - 1) / NORM_MAX_ITERS;   // threads so that 4 iterations cover the row
   t = (t + 63) / 64 * 64;
@@ -304,13 +316,17 @@ VDAMD_API int vdamd_silu_and_mul(void* out, const void* x, long T, int F, int dt
 VDAMD_API int vdamd_embedding(void* out, const int* ids, const void* w, int T, int H, int vocab_start, int rows,
                               int dtype, hipStream_t s) {
   if (T == 0) return 0;
-  if (H % 8 != 0) return -1;
+  if (dtype != DT_BF16 && dtype != DT_F16) return -2;   // (a pure 2-byte copy: one instantiation serves both)
+  if (H % 8 != 0) {
+    hipLaunchKernelGGL(embedding_scalar_kernel<bf16_t>, dim3(T), dim3(H >= 256 ? 256 : 64), 0, s, (bf16_t*)out, ids,
+                       (const bf16_t*)w, H, vocab_start, rows);
+    HIP_LAUNCH_CHECK();
+    return 0;
+  }
   int threads = ((H >> 3) + 63) / 64 * 64;
   if (threads > 256) threads = 256;
-  if (dtype == DT_BF16 || dtype == DT_F16)   // pure 2-byte copy: one instantiation serves both
-    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T), dim3(threads), 0, s, (bf16_t*)out, ids,
-                       (const bf16_t*)w, H, vocab_start, rows);
-  else return -2;
+  hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T), dim3(threads), 0, s, (bf16_t*)out, ids,
+                     (const bf16_t*)w, H, vocab_start, rows);
   HIP_LAUNCH_CHECK();
   return 0;
 }

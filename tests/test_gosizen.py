@@ -64,7 +64,7 @@ def config(layers, width=48, vocab=97, eps=1e-5, loop=None, side=8, cap=12.0):
 
 
 # (the widths of the two low-rank projections of a right half are sizes only the tensors state)
-RANKS = {"varied": (6, 10), "degenerate": (3, 3), "paged": (5, 7), "plain": (4, 4), "wide": (8, 8)}
+RANKS = {"varied": (6, 10), "degenerate": (3, 3), "paged": (5, 7), "plain": (4, 4), "wide": (8, 8), "uneven": (5, 9)}
 
 CONFIGS = {
     # every layer of another shape; a loop over a latent and a parallel layer run three times; a parallel layer in
@@ -95,6 +95,12 @@ CONFIGS = {
     # rows of 64 + 32 values)
     "wide": config([parallel(left(4, 2, 64, 32, 3, 24, 32), right(4, 4, 32, 32, 4), 0.6, 0.5, moe(4, 2, 64)),
                     latent(4, 32, 32, 32, 64, 64, 20, dense(128))], width=128, loop=(0, 2, 2), side=8),
+    # a width, a vocabulary and sizes that are no multiples of 8 (no 16-byte access fits a 16-bit row)
+    "uneven": config([
+        latent(3, 10, 6, 14, 22, 18, 30, moe(5, 2, 30), base=3000.0),
+        parallel(left(3, 1, 20, 12, 3, 45, 10), right(3, 3, 12, 20, 4), 0.8, 0.3, dense(50)),
+        parallel(left(2, 2, 12, 12, 4, 64, 12), right(4, 1, 20, 10, 2), 0.5, 0.7, moe(3, 1, 26))],
+        width=100, vocab=211, loop=(1, 3, 2), side=6, cap=9.0),
 }
 
 

@@ -61,8 +61,9 @@ def test_silu_and_mul(T, F):
                                rtol=2e-2, atol=2e-2)
 
 
-def test_embedding_vocab_shard():
-    w = _rand(1000, 256)
+@pytest.mark.parametrize("width", [256, 100, 7])
+def test_embedding_vocab_shard(width):
+    w = _rand(1000, width)
     ids = torch.tensor([0, 5, 999, 1000, 2500, 1999, 1001], device=DEV, dtype=torch.int32)
     got = ops.embedding(ids, w, vocab_start=1000, masked=True)
     ref = torch_ref.embedding(ids, w, 1000, True)
