@@ -415,8 +415,8 @@ class ScalarRMSNorm(nn.Module):
 
 
 class ResidualRMSNorm(nn.Module):
-    """RMS norm over an fp32 residual stream in fp32 arithmetic, with fp32 gains ``offset + weight`` (``offset`` 1: a
-    weight stored around zero).  ``forward`` returns the model dtype (the input of a projection); ``add`` folds one or
+    """RMS norm over an fp32 residual stream in fp32 arithmetic, with fp32 gains ``offset + weight`` (``offset`` 1: the
+    checkpoint keeps the gain minus one).  ``forward`` returns the model dtype (the input of a projection); ``add`` folds one or
     two sublayer outputs into the stream and hands back the normed sum in the same launch; ``after`` does so for an
     output that is itself RMS-normed with ``post_weight`` before it joins the stream."""
 
