@@ -407,7 +407,7 @@ def test_the_delta_rule_overwrites_and_forgets_and_stale_slots_do_not_show(devic
 
 
 @pytest.mark.parametrize("device,dtype", OP_DEVICES)
-@pytest.mark.parametrize("dim,vdim,heads,qk", [(24, 20, 3, 1), (32, 32, 4, 4), (96, 40, 2, 2), (160, 16, 1, 1)])
+@pytest.mark.parametrize("dim,vdim,heads,qk", [(24, 20, 3, 1), (32, 32, 4, 4), (96, 40, 2, 2), (160, 16, 1, 1), (10, 7, 2, 2), (66, 33, 2, 1)])
 def test_delta_rule_sizes(device, dtype, dim, vdim, heads, qk):
     """Head sizes on both sides of every tiling of the recurrence kernel, value heads sharing query / key heads, two
     sequences in one call (one continuing from a state, one starting)."""
