@@ -95,14 +95,15 @@ template <int P, bool NEAR> __device__ __forceinline__ float parts_sum(float v) 
 }
 
 // grid (tiles of CB = 4 * 64 / P value columns, H, sequences), 4 waves: wave w owns columns w * 64 / P .. of the tile,
-// a lane keeps rows part * R .. part * R + R - 1 of one column of S in registers (P R >= dim).  Two lane layouts.
+// a lane keeps R rows of one column of S in registers (P R >= dim; groups of four rows, dealt to the parts in turn).
+// Two lane layouts.
 // Launches of decoded rows are bound by reading and writing the states: P = 4, parts 16 lanes apart, so that a wave
 // reads 64 bytes of a state row at a time.  Prompt portions are bound by the chain of dependent steps per row (the
 // state cannot be written before r = (gS)^T k is summed over the parts): P = 8 or 16 neighbouring lanes per column,
 // short chains, and the sums stay in the vector unit.  The sequence's rows are walked in chunks of C: q, k, g (all of
 // the head, fp32), v (the tile's columns), b and k.q of a chunk are staged in LDS by the whole workgroup - the next
 // chunk's loads are in flight while the current one is computed, one barrier per chunk - and read back as broadcasts
-// (16-byte reads: a lane's rows are neighbours).
+// (16-byte reads: a group of four rows).
 // x rows hold v (H * vdim) at column v_off; qn / kn [T, G, dim], decay [T, H, dim], bsig [T, 2, H] (sigmoid(beta), then
 // k.q of the head's group) fp32; out [T, H * vdim] fp32; state [slots, H, dim, vdim] fp32.
 template <typename T, int R, int C, int P, bool NEAR>
@@ -128,12 +129,14 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(float* __restrict
   if (n <= 0) return;                               // (the whole workgroup)
   const bool col_ok = col < vdim;
   const int ccol = col_ok ? col : vdim - 1;
-  const int r0 = part * R;
+  // the lane's rows: groups of four, the groups of neighbouring parts side by side (the 16 parts of a column read 256
+  // consecutive bytes of q, k or g at a time: no LDS bank is asked twice)
+  auto row_of = [&](int i) { return ((i >> 2) * P + part) * 4 + (i & 3); };
   float* st = state + (((long)slots[s] * H + h) * dim) * vdim + ccol;
   float S[R];
   const bool fresh = seq_lens[s] - n <= 0;          // the rows start the sequence: whatever the slot holds is not ours
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = (!fresh && r0 + i < dim) ? st[(long)(r0 + i) * vdim] : 0.f;
+  for (int i = 0; i < R; ++i) S[i] = (!fresh && row_of(i) < dim) ? st[(long)row_of(i) * vdim] : 0.f;
 
   // staging: a thread brings 16 bytes of q, of k and of g per pass (all of one row), v and b / k.q element by element
   constexpr int F4 = DP / 4;                        // 16-byte pieces per row and array (a power of two)
@@ -210,9 +213,10 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(float* __restrict
       float kr[R];
 #pragma unroll
       for (int i = 0; i < R; i += 4) {
-        const f32x4 qv = *reinterpret_cast<const f32x4*>(L + r0 + i);
-        const f32x4 kv = *reinterpret_cast<const f32x4*>(L + DP + r0 + i);
-        const f32x4 gv = *reinterpret_cast<const f32x4*>(L + 2 * DP + r0 + i);
+        const int off = ((i >> 2) * P + part) * 4;
+        const f32x4 qv = *reinterpret_cast<const f32x4*>(L + off);
+        const f32x4 kv = *reinterpret_cast<const f32x4*>(L + DP + off);
+        const f32x4 gv = *reinterpret_cast<const f32x4*>(L + 2 * DP + off);
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
           S[i + e] *= gv[e];
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(float* __restrict
   if (col_ok) {
 #pragma unroll
     for (int i = 0; i < R; ++i)
-      if (r0 + i < dim) st[(long)(r0 + i) * vdim] = S[i];
+      if (row_of(i) < dim) st[(long)row_of(i) * vdim] = S[i];
   }
 }
 
