@@ -153,6 +153,21 @@ def normalize_hf_config(cfg: Dict[str, Any]) -> None:
                      ("head_dim", first.get("dim")), ("tie_word_embeddings", False)):
             if cfg.get(k) is None and v is not None:
                 cfg[k] = v
+    if cfg.get("architecture") == "Nalasun" or cfg.get("model_type") == "nalasun":
+        # Nalasun lists its layers one by one as well; its position table bounds a sequence; the logits come from
+        # the embedding table
+        cfg.setdefault("model_type", "nalasun")
+        cfg.setdefault("architectures", ["NalasunForCausalLM"])
+        mixers = [l.get("mixer") or {} for l in cfg.get("layers") or []]
+        first = next((m for l, m in zip(cfg.get("layers") or [], mixers) if l.get("type") == "attention"),
+                     mixers[0] if mixers else {})
+        for k, v in (("hidden_size", cfg.get("width")), ("vocab_size", cfg.get("vocab")),
+                     ("max_position_embeddings", cfg.get("max_positions")), ("num_hidden_layers", len(mixers)),
+                     ("num_attention_heads", first.get("heads", 1)),
+                     ("num_key_value_heads", first.get("kv_heads") or first.get("heads", 1)),
+                     ("head_dim", first.get("dim") or first.get("vdim")), ("tie_word_embeddings", True)):
+            if cfg.get(k) is None and v is not None:
+                cfg[k] = v
     if cfg.get("model_type") == "dbrx":
         # DBRX nests its attention and expert settings
         a, f = cfg.get("attn_config") or {}, cfg.get("ffn_config") or {}

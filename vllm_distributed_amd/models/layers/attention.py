@@ -396,6 +396,41 @@ class WindowBiasAttention(Attention):
         return out.view(t, self.num_heads * self.vdim)
 
 
+class CrossedBiasAttention(WindowBiasAttention):
+    """Causal softmax attention with the logarithmic distance bias of ``WindowBiasAttention`` whose VALUES ARE ITS
+    KEYS as projected (the key rows hold the normed keys, the values the projection itself, so ``vdim = dim`` and
+    there is no value projection) and whose heads exchange their softmax weights: ``weight_h <- sum_g talk[h, g]
+    weight_g``, head ``h`` then applying the mixed weights to the values of its own key / value head.  Computed as
+    ``o_h = sum_g talk[h, g] * (weight_g applied to the values of h's key / value head)``: the attention kernel
+    applies every query head's weights to every value head (fp32 ``[T, H, Hkv, dim]``) and ``ops.mix_heads`` sums.
+    Callers norm q / k and write the cache with ``ops.joint_norm_cache``."""
+
+    def __init__(self, num_heads: int, dim: int, num_kv_heads: int, scale: float, layer_idx: int,
+                 distance_bias: bool = True):
+        super().__init__(num_heads, dim, dim, num_kv_heads, scale, layer_idx, distance_bias=distance_bias, sink=False)
+        self.talk = nn.Parameter(torch.eye(num_heads, dtype=torch.float32), requires_grad=False)
+
+    def forward_cached(self, q: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``q[T, Hq, dim]`` (this step's keys and values already cached) -> ``[T, Hq * dim]`` in ``q``'s dtype."""
+        md = _CTX.attn_metadata
+        t = q.shape[0]
+        if md is None:               # memory-profiling pass: no cache bound
+            return q.new_zeros((t, self.num_heads * self.vdim))
+        out = torch.empty((t, self.num_heads, self.num_kv_heads, self.vdim), dtype=torch.float32, device=q.device)
+        pos = _CTX.positions
+        nd, nb = md.num_decode_tokens, md.num_decodes
+        common = (self.scale, self.bias_scale, self.bias_rate)
+        if nd > 0:
+            ops.crossed_bias_attention(q[:nd], self.k_cache, self.v_cache, md.block_table[:nb],
+                                       md.query_start_loc[:nb + 1], md.seq_lens[:nb], None, pos[:nd], *common, 1,
+                                       out=out[:nd])
+        if md.num_prefills > 0:
+            ops.crossed_bias_attention(q[nd:], self.k_cache, self.v_cache, md.block_table[nb:],
+                                       md.prefill_query_start_loc, md.seq_lens[nb:], md.prefill_token_rows(pos),
+                                       pos[nd:], *common, md.max_prefill_query_len, out=out[nd:])
+        return ops.mix_heads(out, self.talk, q.dtype)
+
+
 class ScalarRMSNorm(nn.Module):
     """RMS norm whose gain is a single number for all coordinates, in fp32 arithmetic; ``forward`` returns the
     model dtype (the input of a projection), ``residual_add`` folds a sublayer's output into the fp32 residual

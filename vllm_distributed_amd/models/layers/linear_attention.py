@@ -1,4 +1,5 @@
-"""Linear attention with a recurrent state per request: a decay per head, or the gated delta rule.
+"""Linear attention with a recurrent state per request: a decay per head, the gated delta rule, or a state-space
+recurrence whose decay depends on the token.
 
 Per head ``S_t = decay[h] * S_(t-1) + k_t v_t^T`` and ``o_t = S_t^T q_t``: no softmax, no cache that grows with the
 sequence.  What a request carries from token to token is the ``dim x vdim`` matrix ``S`` of every head, in fp32, one
@@ -79,3 +80,39 @@ class GatedDeltaRule(nn.Module):
         return ops.gated_delta_rule(x, self.heads, self.qk_heads, self.dim, self.vdim, beta, dt, self.dt_bias,
                                     self.a_log, state, md.state_slots, md.query_start_loc, md.seq_lens, self.norm_eps,
                                     md.max_query_len)
+
+
+class SelectiveStateSpace(nn.Module):
+    """A state-space recurrence in its dual (attention-like) form: per head an ``n_state x vdim`` fp32 state with
+    ``S <- exp(-exp(a_log[h]) * d) * S + d * B u^T`` and ``y = S^T C + d_skip[h] * u``, where the step size
+    ``d = softplus(dt + dt_bias[h])`` comes from the token (no clamp); ``heads`` heads share ``groups`` B / C vectors
+    in runs of neighbours.  The state tensors are ``layers.short_conv.SlotState`` objects the caller owns;
+    ``forward`` reads ``[u | B | C]`` from the leading columns of ``x`` and returns the fp32 heads
+    ``[T, heads * vdim]`` side by side.  ``skip`` False: no ``d_skip`` term."""
+
+    def __init__(self, heads: int, groups: int, vdim: int, n_state: int, layer_idx: int, skip: bool = True):
+        super().__init__()
+        if groups < 1 or heads % groups:
+            raise ValueError(f"layer {layer_idx}: {heads} heads do not divide over {groups} B / C groups")
+        self.heads, self.groups, self.vdim, self.n_state = heads, groups, vdim, n_state
+        self.layer_idx = layer_idx
+        f32 = torch.float32
+        self.a_log = nn.Parameter(torch.zeros(heads, dtype=f32), requires_grad=False)
+        self.dt_bias = nn.Parameter(torch.zeros(heads, dtype=f32), requires_grad=False)
+        self.d_skip = nn.Parameter(torch.zeros(heads, dtype=f32), requires_grad=False) if skip else None
+
+    @property
+    def channels(self) -> int:
+        """Columns ``forward`` reads: ``[u | B | C]``."""
+        return self.heads * self.vdim + 2 * self.groups * self.n_state
+
+    def per_slot_shape(self) -> Tuple[int, int, int]:
+        return (self.heads, self.n_state, self.vdim)
+
+    def forward(self, x: torch.Tensor, dt: torch.Tensor, state: Optional[torch.Tensor]) -> torch.Tensor:
+        md = get_forward_context().attn_metadata
+        if md is None or state is None:   # memory-profiling pass: no state bound
+            return x.new_zeros((x.shape[0], self.heads * self.vdim), dtype=torch.float32)
+        return ops.selective_scan(x, dt, self.heads, self.groups, self.vdim, self.n_state, self.a_log, self.dt_bias,
+                                  self.d_skip, state, md.state_slots, md.query_start_loc, md.seq_lens,
+                                  md.max_query_len)

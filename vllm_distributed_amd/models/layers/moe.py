@@ -595,3 +595,121 @@ class BiasedTopKMoE(FusedMoE):
                 acc.index_add_(0, rows, self._expert_mlp(eid, x.index_select(0, rows)).float() * wts[seg].unsqueeze(1))
             start += n
         return acc.to(x.dtype)
+
+
+class GatedMLP(nn.Module):
+    """One feed-forward of the gated form ``down(silu(gate(x)) * up(x))``, gate and up as one fused projection; no
+    biases."""
+
+    def __init__(self, hidden: int, inter: int, dtype: torch.dtype):
+        super().__init__()
+        self.inter = inter
+        self.w13 = nn.Parameter(torch.empty(2 * inter, hidden, dtype=dtype), requires_grad=False)
+        self.w2 = nn.Parameter(torch.empty(hidden, inter, dtype=dtype), requires_grad=False)
+        self.w13.weight_loader = self._load_w13
+
+    def _load_w13(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        param.data.narrow(0, int(shard_id) * self.inter, self.inter).copy_(materialize(w))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.linear(ops.silu_and_mul(ops.linear(x, self.w13)), self.w2)
+
+
+class ScoredTopKMoE(FusedMoE):
+    """Routed experts of the gated form ``down(silu(gate(x)) * up(x))`` behind a router whose outputs are scored one
+    by one: ``score = sigmoid(router(x))``, the ``top_k`` largest scores are chosen and ARE the weights, times
+    ``route_scale``, not renormalised.  ``shared_inter > 0``: an expert of the same form that every token uses, whose
+    output ``forward`` returns beside the routed sum (the caller adds both to its residual stream in one launch).
+
+    The router is fp32 (product and scores).  On the GPU in 16-bit types the experts run as two grouped GEMMs over
+    expert-sorted rows, their reduction dimensions zero-padded to the kernels' 128-deep tiles; elsewhere (fp32, CPU)
+    one after the other on the library GEMM."""
+    custom_routing = True
+
+    def __init__(self, hidden: int, inter: int, num_experts: int, top_k: int, dtype: torch.dtype,
+                 route_scale: float = 1.0, shared_inter: int = 0):
+        super().__init__(hidden, inter, num_experts, top_k, False, dtype, expert_parallel=False, allocate_experts=False)
+        if self.tp > 1:
+            raise NotImplementedError("ScoredTopKMoE runs unsharded")
+        if not 1 <= top_k <= num_experts:
+            raise ValueError(f"top {top_k} of {num_experts} experts")
+        self.quant = None
+        self.route_scale = float(route_scale)
+        self.gate = ReplicatedLinear(hidden, num_experts, False, dtype, quant=False)
+        self.h_pad, self.i_pad = _ceil128(hidden), _ceil128(inter)
+        # [gate rows ; up rows] (each padded to i_pad rows) x (reduction padded to h_pad); [hidden, i_pad]
+        self.w13 = nn.Parameter(torch.zeros(num_experts, 2 * self.i_pad, self.h_pad, dtype=dtype), requires_grad=False)
+        self.w2 = nn.Parameter(torch.zeros(num_experts, hidden, self.i_pad, dtype=dtype), requires_grad=False)
+        self.w13.weight_loader = self._load_w13
+        self.w2.weight_loader = self._load_w2
+        self.shared = GatedMLP(hidden, shared_inter, dtype) if shared_inter else None
+
+    def _load_w13(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        e, which = shard_id                  # which: 0 = gate, 1 = up
+        dst = param.data[e, which * self.i_pad:(which + 1) * self.i_pad]
+        dst.zero_()                          # (the padding included: the loader poisons fresh parameters)
+        dst[:self.inter, :self.hidden].copy_(materialize(w))
+
+    def _load_w2(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
+        e, _ = shard_id
+        param.data[e].zero_()
+        param.data[e, :, :self.inter].copy_(materialize(w))
+
+    def router_logits(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.linear_f32(x, self.gate.weight)
+
+    def route(self, logits: torch.Tensor):
+        val, topi = torch.sigmoid(logits.float()).topk(self.top_k, dim=-1)
+        return val * self.route_scale, topi
+
+    def _pad(self, x: torch.Tensor) -> torch.Tensor:
+        return x if self.h_pad == self.hidden else F.pad(x, (0, self.h_pad - self.hidden))
+
+    def _expert_mlp(self, e: int, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(ops.silu_and_mul(F.linear(self._pad(x), self.w13[e])), self.w2[e])
+
+    def _grouped_tile_rows(self, x: torch.Tensor) -> int:
+        if not (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and x.dim() == 2 and ops.hip_available()):
+            return 0
+        if self.num_experts > 512 or self.top_k > 16 or self.hidden % 16:
+            return 0
+        avg = x.shape[0] * self.top_k / max(1, self.num_experts)
+        if avg > envs.VDAMD_MOE_GROUPED_MAX_ROWS * 2 and not torch.cuda.is_current_stream_capturing():
+            return 0
+        for rows in (16, 32, 64, 128):
+            if avg <= rows:
+                return rows
+        return 128
+
+    def decode_capturable(self, dtype: torch.dtype) -> bool:
+        """Whether a decode step of this block runs without a host synchronisation (the grouped path)."""
+        return (dtype in (torch.bfloat16, torch.float16) and self.hidden % 16 == 0 and self.num_experts <= 512
+                and self.top_k <= 16)
+
+    def forward(self, x: torch.Tensor, reduce: bool = True, staged: bool = False, deferred: bool = False):
+        """Returns ``(routed sum, shared expert's output or None)``."""
+        logits = self.router_logits(x)
+        shared = self.shared(x) if self.shared is not None else None
+        tile_rows = self._grouped_tile_rows(x)
+        if tile_rows:
+            topw, topi = ops.moe_topk_grouped(logits, None, self.top_k, 1, 1, True, False, False, self.route_scale)
+            src_row, inv, tiles = ops.moe_align_fused(topi, self.num_experts, tile_rows, 0, -1)
+            xs = self._pad(x).index_select(0, src_row)
+            h = ops.grouped_linear(xs, tiles, tile_rows, weight=self.w13)
+            y = ops.grouped_linear(ops.silu_and_mul(h), tiles, tile_rows, weight=self.w2)
+            return ops.moe_combine(y, topw, topi, inv, 0, -1), shared
+        topw, topi = self.route(logits)
+        acc = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        flat_e = topi.reshape(-1)
+        order = flat_e.argsort(stable=True)
+        counts = torch.bincount(flat_e, minlength=self.num_experts).tolist()
+        tok = order // self.top_k
+        wts = topw.reshape(-1)[order]
+        start = 0
+        for eid, n in enumerate(counts):
+            if n:
+                seg = slice(start, start + n)
+                rows = tok[seg]
+                acc.index_add_(0, rows, self._expert_mlp(eid, x.index_select(0, rows)).float() * wts[seg].unsqueeze(1))
+            start += n
+        return acc.to(x.dtype), shared

@@ -17,9 +17,10 @@ import torch.nn as nn
 
 class ShortConv(nn.Module):
     """``weight[channels, taps]`` for the leading ``channels`` columns of a fused projection; the checkpoint may
-    hold it in pieces (one per projection), loaded into consecutive row ranges."""
+    hold it in pieces (one per projection), loaded into consecutive row ranges.  ``bias``: one fp32 number per
+    channel, added to the convolution's sum."""
 
-    def __init__(self, piece_sizes: Sequence[int], taps: int, dtype: torch.dtype):
+    def __init__(self, piece_sizes: Sequence[int], taps: int, dtype: torch.dtype, bias: bool = False):
         super().__init__()
         self.piece_sizes = list(piece_sizes)
         self.channels, self.taps = sum(self.piece_sizes), int(taps)
@@ -27,6 +28,7 @@ class ShortConv(nn.Module):
             raise ValueError("a convolution needs at least one tap")
         self.weight = nn.Parameter(torch.empty(self.channels, self.taps, dtype=dtype), requires_grad=False)
         self.weight.weight_loader = self.load_piece          # type: ignore[attr-defined]
+        self.bias = nn.Parameter(torch.zeros(self.channels, dtype=torch.float32), requires_grad=False) if bias else None
         self.state: Optional[torch.Tensor] = None
         self.dtype = dtype
         # what the kernels read: the same numbers tap-major, ``[taps, channels]`` (the taps of neighbouring

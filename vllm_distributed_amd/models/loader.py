@@ -57,6 +57,9 @@ def _weight_shapes(c: dict, arch: str) -> Dict[str, Tuple[int, ...]]:
     if arch in ("GosizenForCausalLM", "Gosizen"):
         from .gosizen import weight_shapes
         return weight_shapes(c)
+    if arch in ("NalasunForCausalLM", "Nalasun"):
+        from .nalasun import weight_shapes
+        return weight_shapes(c)
     if arch == "MedusaModel":
         h = c["hidden_size"]
         out = {}
@@ -468,6 +471,10 @@ def dummy_weights_iterator(mc: ModelConfig, device: torch.device,
             continue
         if mc.architecture in ("GosizenForCausalLM", "Gosizen"):
             from .gosizen import random_weight
+            yield name, random_weight(name, shape, gen, device, dtype)
+            continue
+        if mc.architecture in ("NalasunForCausalLM", "Nalasun"):
+            from .nalasun import random_weight
             yield name, random_weight(name, shape, gen, device, dtype)
             continue
         if awq and _QUANTIZED_LINEAR.search(name) and shape[1] % g == 0 and shape[0] % 8 == 0:

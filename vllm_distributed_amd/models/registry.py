@@ -75,6 +75,11 @@ _MODELS: Dict[str, Tuple[str, str]] = {
     # chunked attention over convolved keys beside the gated delta rule; a block of layers that runs several times
     "GosizenForCausalLM": ("gosizen", "GosizenForCausalLM"),
     "Gosizen": ("gosizen", "GosizenForCausalLM"),
+    # fp32 residual stream and learned positions; a convolution in front of every mixer; attention whose values are
+    # its keys and whose heads mix their softmax weights, the gated delta rule, a state-space recurrence; experts
+    # weighted by sigmoid scores
+    "NalasunForCausalLM": ("nalasun", "NalasunForCausalLM"),
+    "Nalasun": ("nalasun", "NalasunForCausalLM"),
     # draft heads of speculative decoding (never a served model by themselves; worker/draft_model.py)
     "EagleLlamaForCausalLM": ("spec_heads", "EagleLlamaForCausalLM"),
     "Eagle3LlamaForCausalLM": ("spec_heads", "Eagle3LlamaForCausalLM"),
@@ -87,7 +92,7 @@ _MODELS: Dict[str, Tuple[str, str]] = {
 # architectures whose layers keep per-request state besides the KV cache (convolution tails, recurrences): a cached
 # prefix's blocks do not bring that state back, so prefix reuse is off for them
 _KEEPS_REQUEST_STATE = {"TavulixForCausalLM", "Tavulix", "KabapelForCausalLM", "Kabapel", "GosizenForCausalLM",
-                        "Gosizen"}
+                        "Gosizen", "NalasunForCausalLM", "Nalasun"}
 
 
 def keeps_request_state(arch: str) -> bool:

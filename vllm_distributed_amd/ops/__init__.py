@@ -814,13 +814,15 @@ def gelu(x, tanh: bool):
 
 
 def short_conv_act(x, channels: int, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions,
-                   silu: bool, has_prefill: bool = True):
+                   silu: bool, has_prefill: bool = True, bias=None, residual: bool = False):
     """Causal convolution over time (tap-major ``conv_weight[taps, channels]``, per-request state) of the first
-    ``channels`` columns of a fused projection, through SiLU when asked; see ``torch_ref.short_conv_act``."""
+    ``channels`` columns of a fused projection, plus ``bias``, through SiLU when asked, plus the input itself with
+    ``residual``; see ``torch_ref.short_conv_act``."""
     if _use_hip(x):
         return _hip.short_conv_act(x, channels, conv_weight, state, slots, query_start_loc, seq_lens, token_seq,
-                                   positions, silu, has_prefill)
-    return torch_ref.short_conv_act(x, channels, conv_weight, state, slots, query_start_loc, seq_lens, silu)
+                                   positions, silu, has_prefill, bias, residual)
+    return torch_ref.short_conv_act(x, channels, conv_weight, state, slots, query_start_loc, seq_lens, silu, bias,
+                                    residual)
 
 
 def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, beta, dt, dt_bias, a_log, state,
@@ -832,3 +834,59 @@ def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, 
                                      query_start_loc, seq_lens, norm_eps, max_query_len)
     return torch_ref.gated_delta_rule(x, num_heads, num_qk_heads, dim, vdim, beta, dt, dt_bias, a_log, state, slots,
                                       query_start_loc, seq_lens, norm_eps)
+
+
+# ------------------------------------------------ selective state-space scan, gate in front of a grouped norm,
+# ------------------------------------------------ q / k normed over all heads with values = keys, crossed value
+# ------------------------------------------------ heads and mixed head weights
+def selective_scan(x, dt, num_heads: int, groups: int, vdim: int, n_state: int, a_log, dt_bias, d_skip, state, slots,
+                   query_start_loc, seq_lens, max_query_len: int = 0):
+    """A state-space recurrence with a data-dependent decay per head and a per-request fp32 state; see
+    ``torch_ref.selective_scan``."""
+    if _use_hip(x):
+        return _hip.selective_scan(x, dt, num_heads, groups, vdim, n_state, a_log, dt_bias, d_skip, state, slots,
+                                   query_start_loc, seq_lens, max_query_len)
+    return torch_ref.selective_scan(x, dt, num_heads, groups, vdim, n_state, a_log, dt_bias, d_skip, state, slots,
+                                    query_start_loc, seq_lens)
+
+
+def act_gate_group_norm(y, gate, weight, eps: float, group: int, out_dtype):
+    """``rms_norm_by_groups(y * silu(gate)) * weight``; see ``torch_ref.act_gate_group_norm``."""
+    if _use_hip(y):
+        return _hip.act_gate_group_norm(y, gate, weight, eps, group, out_dtype)
+    return torch_ref.act_gate_group_norm(y, gate, weight, eps, group, out_dtype)
+
+
+def joint_norm_cache(x, num_heads: int, num_kv_heads: int, dim: int, q_norm, k_norm, eps: float, positions,
+                     temp_coef: float, temp_every: int, k_cache, v_cache, slot_mapping):
+    """q and k normed over all their heads at once, the query's position factor, normed k into the key rows and the
+    projected k into the values; see ``torch_ref.joint_norm_cache``."""
+    if _use_hip(x):
+        return _hip.joint_norm_cache(x, num_heads, num_kv_heads, dim, q_norm, k_norm, eps, positions, temp_coef,
+                                     temp_every, k_cache, v_cache, slot_mapping)
+    return torch_ref.joint_norm_cache(x, num_heads, num_kv_heads, dim, q_norm, k_norm, eps, positions, temp_coef,
+                                      temp_every, k_cache, v_cache, slot_mapping)
+
+
+def crossed_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
+                           scale: float, bias_scale, bias_rate, max_query_len: int = 0, out=None):
+    """Every query head's softmax weights on every value head, fp32 ``[T, Hq, Hkv, Dv]``; see
+    ``torch_ref.crossed_bias_attention``."""
+    if _use_hip(q):
+        attention_calls["hip"] += 1
+        return _hip.window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq,
+                                          positions, scale, 0.0, 0, 0, bias_scale, bias_rate, None, None,
+                                          max_query_len, out, 0, crossed=True)
+    res = torch_ref.crossed_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, scale,
+                                           bias_scale, bias_rate)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def mix_heads(o, talk, out_dtype):
+    """Heads mixed by ``talk[H, H]`` over crossed attention outputs; see ``torch_ref.mix_heads``."""
+    if _use_hip(o):
+        return _hip.mix_heads(o, talk, out_dtype)
+    return torch_ref.mix_heads(o, talk, out_dtype)

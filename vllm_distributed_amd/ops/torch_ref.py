@@ -843,11 +843,19 @@ def sigmoid_mul(o: torch.Tensor, gate: torch.Tensor, scale: float = 1.0, out: Op
 
 
 def short_conv_act(x: torch.Tensor, channels: int, conv_weight: torch.Tensor, state: torch.Tensor, slots: torch.Tensor,
-                   query_start_loc: torch.Tensor, seq_lens: torch.Tensor, silu: bool) -> torch.Tensor:
-    """``short_conv`` over the first ``channels`` columns of ``x`` (the state moves on), through SiLU when ``silu``;
+                   query_start_loc: torch.Tensor, seq_lens: torch.Tensor, silu: bool,
+                   bias: Optional[torch.Tensor] = None, residual: bool = False) -> torch.Tensor:
+    """``short_conv`` over the first ``channels`` columns of ``x`` (the state moves on), plus ``bias[channels]``,
+    through SiLU when ``silu``; with ``residual`` the input itself is added at the end (``x + conv(x)``);
     ``[T, channels]`` in ``x``'s dtype."""
     y = short_conv(x[:, :channels], conv_weight, state, slots, query_start_loc, seq_lens)
-    return (F.silu(y) if silu else y).to(x.dtype)
+    if bias is not None:
+        y = y + bias.float()
+    if silu:
+        y = F.silu(y)
+    if residual:
+        y = y + x[:, :channels].float()
+    return y.to(x.dtype)
 
 
 def gated_delta_rule(x: torch.Tensor, num_heads: int, num_qk_heads: int, dim: int, vdim: int, beta: torch.Tensor,
@@ -887,3 +895,118 @@ def gated_delta_rule(x: torch.Tensor, num_heads: int, num_qk_heads: int, dim: in
             out[r] = torch.einsum("hkv,hk->hv", st, q[r])
         state[sl[i]] = st.to(state.dtype)
     return out.reshape(t, h * vdim)
+
+
+# ------------------------------------------------ selective state-space scan, gate in front of a grouped norm,
+# ------------------------------------------------ q / k normed over all heads with values = keys, crossed value
+# ------------------------------------------------ heads and mixed head weights
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, num_heads: int, groups: int, vdim: int, n_state: int,
+                   a_log: torch.Tensor, dt_bias: torch.Tensor, d_skip: Optional[torch.Tensor], state: torch.Tensor,
+                   slots: torch.Tensor, query_start_loc: torch.Tensor, seq_lens: torch.Tensor) -> torch.Tensor:
+    """A state-space recurrence with one data-dependent decay per head over the packed rows ``x[T, C]`` =
+    ``[u (H * vdim) | B (G * N) | C (G * N)]``; head ``h`` reads B / C group ``h // (H / G)``.  Per row
+    ``d = softplus(dt[t, h] + dt_bias[h])`` (no clamp), ``S <- exp(-exp(a_log[h]) * d) * S + d * B u^T`` (``S`` is
+    ``N x vdim``), ``y = S^T C + d_skip[h] * u``.  ``S`` is ``state[slots[i]]`` (``[slots, H, N, vdim]`` fp32) for
+    sequence ``i``, taken as zero when the rows start at position 0 whatever the slot held, and left holding the state
+    after the sequence's last row.  fp32 arithmetic; returns fp32 ``[T, H * vdim]``."""
+    t, h, g, n = x.shape[0], num_heads, groups, n_state
+    inner = h * vdim
+    xf = x[:, :inner + 2 * g * n].float()
+    u = xf[:, :inner].reshape(t, h, vdim)
+    bm = xf[:, inner:inner + g * n].reshape(t, g, n).repeat_interleave(h // g, dim=1)
+    cm = xf[:, inner + g * n:].reshape(t, g, n).repeat_interleave(h // g, dim=1)
+    d = F.softplus(dt[:t].float() + dt_bias.float().view(1, h), threshold=30.0)
+    decay = torch.exp(-torch.exp(a_log.float()).view(1, h) * d)
+    out = torch.zeros((t, h, vdim), dtype=torch.float32, device=x.device)
+    qsl, sls, sl = query_start_loc.tolist(), seq_lens.tolist(), slots.tolist()
+    for i, n_ctx in enumerate(sls):
+        s, e = qsl[i], qsl[i + 1]
+        if e == s:
+            continue
+        st = state[sl[i]].float().clone() if n_ctx - (e - s) > 0 else torch.zeros_like(state[sl[i]], dtype=torch.float32)
+        for r in range(s, e):
+            st = decay[r].view(h, 1, 1) * st + (d[r].view(h, 1) * bm[r]).unsqueeze(2) * u[r].unsqueeze(1)
+            out[r] = torch.einsum("hnv,hn->hv", st, cm[r])
+        state[sl[i]] = st.to(state.dtype)
+    if d_skip is not None:
+        out = out + d_skip.float().view(1, h, 1) * u
+    return out.reshape(t, inner)
+
+
+def act_gate_group_norm(y: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, group: int,
+                        out_dtype: torch.dtype) -> torch.Tensor:
+    """``y * silu(gate)`` first, then the RMS norm of each run of ``group`` values (``group`` 0: whole rows) times
+    ``weight`` (one gain per column), in fp32 arithmetic; ``[T, N]`` in ``out_dtype``."""
+    z = y.float() * F.silu(gate.float())
+    g = z.unflatten(-1, (-1, group)) if group > 0 else z.unsqueeze(-2)
+    g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+    return (g.flatten(-2) * weight.float()).to(out_dtype)
+
+
+def joint_norm_cache(x: torch.Tensor, num_heads: int, num_kv_heads: int, dim: int, q_norm: torch.Tensor,
+                     k_norm: torch.Tensor, eps: float, positions: torch.Tensor, temp_coef: float, temp_every: int,
+                     k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                     slot_mapping: Optional[torch.Tensor]) -> torch.Tensor:
+    """What lies between the fused projection ``x[T, >= (H + Hkv) * dim]`` = ``[q | k]`` and the attention of a layer
+    whose values are its keys: the RMS norm of q over ALL heads at once with ``q_norm[H * dim]`` (and of k with
+    ``k_norm[Hkv * dim]``), q times ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)`` at position ``p``
+    (``temp_every`` 0: no such factor), normed k into the key rows ``k_cache[blocks, Hkv, block, dim]`` and k AS
+    PROJECTED into the values ``v_cache[blocks, Hkv, block / 8, dim, 8]``.  Returns ``q[T, H, dim]`` in ``x``'s
+    dtype."""
+    t = x.shape[0]
+    qs, ks = num_heads * dim, num_kv_heads * dim
+    xf = x[:, :qs + ks].float()
+    q, k = xf[:, :qs], xf[:, qs:]
+    qn = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()
+    kn = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm.float()
+    if temp_every > 0:
+        p = positions[:t].long()
+        qn = qn * (1.0 + temp_coef * torch.log(torch.div(p + 1, temp_every, rounding_mode="floor").float() + 1.0)).unsqueeze(1)
+    if k_cache is not None:
+        bs = k_cache.shape[2]
+        valid = slot_mapping[:t] >= 0
+        sm = slot_mapping[:t][valid].long()
+        blk, off = sm // bs, sm % bs
+        k_cache[blk, :, off, :] = kn[valid].reshape(-1, num_kv_heads, dim).to(k_cache.dtype)
+        v_cache[blk, :, off // V_GROUP, :, off % V_GROUP] = k[valid].reshape(-1, num_kv_heads, dim).to(v_cache.dtype)
+    return qn.reshape(t, num_heads, dim).to(x.dtype)
+
+
+def crossed_bias_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                           query_start_loc: torch.Tensor, seq_lens: torch.Tensor, scale: float,
+                           bias_scale: Optional[torch.Tensor], bias_rate: Optional[torch.Tensor]) -> torch.Tensor:
+    """Causal softmax attention as ``window_bias_attention`` (no window, cap, sink or gate) in which every query
+    head's weights are applied to the values of EVERY key / value head: fp32 ``[T, Hq, Hkv, Dv]``, entry
+    ``[t, h, c]`` = ``sum_j weight_h(t, j) v_c(j)``."""
+    t, hq, d = q.shape
+    hkv, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    g = hq // hkv
+    out = torch.zeros((t, hq, hkv, dv), dtype=torch.float32, device=q.device)
+    qsl, sls = query_start_loc.tolist(), seq_lens.tolist()
+    for i, sl in enumerate(sls):
+        s, e = qsl[i], qsl[i + 1]
+        ql = e - s
+        if ql == 0:
+            continue
+        blocks = block_table[i, :(sl + bs - 1) // bs].long()
+        k = k_cache[blocks].permute(1, 0, 2, 3).reshape(hkv, -1, d)[:, :sl].float().repeat_interleave(g, dim=0)
+        v = v_cache[blocks].permute(1, 0, 2, 4, 3).reshape(hkv, -1, dv)[:, :sl].float()
+        sc = torch.matmul(q[s:e].float().transpose(0, 1), k.transpose(1, 2)) * scale
+        qpos = torch.arange(sl - ql, sl, device=q.device).unsqueeze(1)
+        kpos = torch.arange(sl, device=q.device).unsqueeze(0)
+        if bias_scale is not None:
+            dist = (qpos - kpos).clamp(min=0).float()
+            sc = sc - bias_scale.float().view(-1, 1, 1) * torch.log1p(bias_rate.float().view(-1, 1, 1) * dist)
+        p = torch.softmax(sc.masked_fill(kpos > qpos, float("-inf")), -1)
+        out[s:e] = torch.einsum("hqk,ckd->qhcd", p, v)
+    return out
+
+
+def mix_heads(o: torch.Tensor, talk: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """``o[T, H, Hkv, Dv]`` (head ``g``'s weights on value head ``c``) and ``talk[H, H]``: head ``h`` gets
+    ``sum_g talk[h, g] * o[t, g, h // (H / Hkv)]``, which is what mixing the heads' softmax weights by ``talk`` and
+    applying them to head ``h``'s own values gives.  fp32 arithmetic; ``[T, H * Dv]`` in ``out_dtype``."""
+    t, h, c, dv = o.shape
+    own = torch.arange(h, device=o.device) // (h // c)
+    picked = o.float()[:, :, own, :]                                # [T, g, h, Dv]
+    return torch.einsum("hg,tghd->thd", talk.float(), picked).reshape(t, h * dv).to(out_dtype)
