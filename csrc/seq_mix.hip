@@ -500,8 +500,8 @@ __global__ void conv_state_update_kernel(const T* __restrict__ x, long x_stride,
   for (int k = 0; k < R; ++k) stf(st + (long)k * C + c, keep[k]);
 }
 
-// The convolution alone (no head structure): out[t, c] = act(sum_j w[j, c] * u[t - taps + 1 + j, c]) for the first C
-// columns of x, history from the step's own rows or the state slot as above.  One thread per (row, channel); the 16-bit
+// The convolution alone (no head structure): out[t, c] = act(bias[c] + sum_j w[j, c] * u[t - taps + 1 + j, c]) for the
+// first C columns of x (plus u[t, c] itself with `residual`), history from the step's own rows or the state slot as above.  One thread per (row, channel); the 16-bit
 // variant gives a thread 8 neighbouring channels (16-byte accesses).  A sequence's only row moves its state on here.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void short_conv_act_kernel(T* __restrict__ out, long out_stride, const T* __restrict__ x,
@@ -509,7 +509,8 @@ __global__ __launch_bounds__(256) void short_conv_act_kernel(T* __restrict__ out
                                                              const int* __restrict__ slots, const int* __restrict__ qsl,
                                                              const int* __restrict__ seq_lens,
                                                              const int* __restrict__ token_seq,
-                                                             const int* __restrict__ positions, int C, int taps, int silu) {
+                                                             const int* __restrict__ positions, int C, int taps, int silu,
+                                                             const float* __restrict__ bias, int residual) {
   constexpr int W = VEC ? 8 : 1;
   const int t = blockIdx.x;
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * W;
@@ -521,9 +522,9 @@ __global__ __launch_bounds__(256) void short_conv_act_kernel(T* __restrict__ out
   const int R = taps - 1;
   T* st = state + (long)slots[s] * (R > 0 ? R : 1) * C;
   const bool own_state = (n == 1) && R > 0;
-  float acc[W];
+  float acc[W], cur[W];
 #pragma unroll
-  for (int e = 0; e < W; ++e) acc[e] = 0.f;
+  for (int e = 0; e < W; ++e) { acc[e] = bias ? bias[c + e] : 0.f; cur[e] = 0.f; }
   for (int j = 0; j < taps; ++j) {
     const int back = taps - 1 - j;
     const int p = pos - back;
@@ -539,18 +540,23 @@ __global__ __launch_bounds__(256) void short_conv_act_kernel(T* __restrict__ out
       }
       if (own_state && j >= 1) st8<T>(st + (long)(j - 1) * C + c, u);       // (row j - 1 was read one turn earlier)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += (float)wv[e] * (float)u[e];
+      for (int e = 0; e < 8; ++e) { acc[e] += (float)wv[e] * (float)u[e]; cur[e] = (float)u[e]; }
     } else {
       float u = 0.f;
       if (p >= chunk_start && p >= 0) u = ldf(x + (long)(t - back) * x_stride + c);
       else if (p >= 0) u = ldf(st + (long)(R - (chunk_start - p)) * C + c);
       if (own_state && j >= 1) stf(st + (long)(j - 1) * C + c, u);
       acc[0] += ldf(w + (long)j * C + c) * u;
+      cur[0] = u;
     }
   }
   if (silu) {
 #pragma unroll
     for (int e = 0; e < W; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
+  }
+  if (residual) {                               // (the last tap's input is the row itself)
+#pragma unroll
+    for (int e = 0; e < W; ++e) acc[e] += cur[e];
   }
   if constexpr (VEC) {
     typename Vec8<T>::type o;
@@ -575,6 +581,8 @@ struct AttnArgs {
   int T, H, G, D, Dv, block_size, window, keep_first;
   float scale, softcap;
   int chunk;                        // > 0: a query sees only the keys of its own block of `chunk` positions
+  int cross;                        // 1: every query head's weights are applied to the values of EVERY key / value head,
+                                    // out is fp32 [T, H, G, Dv] (blockIdx.y then counts (key head, value head) pairs)
 };
 
 template <typename T, bool VEC> struct RowDot;
@@ -616,7 +624,9 @@ constexpr int ATTN_V_PER_LANE = 8;          // Dv <= 512
 template <typename T, bool VEC>
 __global__ void window_bias_attention_kernel(AttnArgs a) {
   extern __shared__ float lds[];
-  const int t = blockIdx.x, g = blockIdx.y;
+  const int t = blockIdx.x;
+  const int g = a.cross ? blockIdx.y / a.G : blockIdx.y;          // key head
+  const int gv = a.cross ? blockIdx.y % a.G : g;                  // value head
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int qpg = a.H / a.G;
   const int hl = blockIdx.z * nwaves + wave;
@@ -657,7 +667,7 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
       sc = RowDot<T, VEC>::run(kc + row * a.D, sq, a.D) * a.scale;
       if (a.softcap > 0.f) sc = a.softcap * tanhf(sc / a.softcap);
       if (a.bias_scale) sc -= r1 * log1pf(r2 * (float)(pos - j));
-      vrow = (((blk * a.G + g) * (a.block_size >> 3) + ((j % a.block_size) >> 3)) * (long)a.Dv) * 8 + (j & 7);
+      vrow = (((blk * a.G + gv) * (a.block_size >> 3) + ((j % a.block_size) >> 3)) * (long)a.Dv) * 8 + (j & 7);
     }
     const float m_new = fmaxf(m, wave_max(sc));
     const float p = f < total ? expf(sc - m_new) : 0.f;
@@ -702,6 +712,17 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
     const float gv = ldf((const T*)a.gate + (long)t * a.gate_stride + h);
     mul *= 1.0f / (1.0f + expf(-gv));
   }
+  if (a.cross) {
+    float* o = (float*)a.out + (((long)t * a.H + h) * a.G + gv) * a.Dv;
+    if (kp == 0) {
+#pragma unroll
+      for (int i = 0; i < ATTN_V_PER_LANE; ++i) {
+        const int c = cl0 + i * cw;
+        if (c < a.Dv) o[c] = acc[i] * mul;
+      }
+    }
+    return;
+  }
   T* o = (T*)a.out + ((long)t * a.H + h) * a.Dv;
   if (kp == 0) {
 #pragma unroll
@@ -734,7 +755,9 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   const int s = blockIdx.z;
   const int qpg = a.H / a.G;
   const int hchunks = (qpg + hp - 1) / hp;
-  const int g = blockIdx.y / hchunks, hc = blockIdx.y % hchunks;
+  const int gy = blockIdx.y / hchunks, hc = blockIdx.y % hchunks;
+  const int g = a.cross ? gy / a.G : gy;          // key head
+  const int gv = a.cross ? gy % a.G : g;          // value head
   const int tw = nwaves / kw;                     // waves over tokens
   const int wt = wave / kw, wk = wave % kw;
   const int q0 = qsl[s], n_tok = qsl[s + 1] - q0;
@@ -822,7 +845,7 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     const int vkey = min(base + 8 * g4, p_last) & ~7;
     split(vkey, bi_v, off_v);
     const long blk_v = bt[bi_v];
-    const T* vp = vc + (((blk_v * a.G + g) * bs8 + (off_v >> 3)) * (long)DV + r16) * 8;
+    const T* vp = vc + (((blk_v * a.G + gv) * bs8 + (off_v >> 3)) * (long)DV + r16) * 8;
     V8 vf[VT];
 #pragma unroll
     for (int c = 0; c < VT; ++c) vf[c] = ld8<T>(vp + (long)c * 128);
@@ -920,6 +943,12 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   if (a.gate) {
     const float gv = (float)((const T*)a.gate)[trow * a.gate_stride + h];
     mul *= 1.0f / (1.0f + expf(-gv));
+  }
+  if (a.cross) {
+    float* o = (float*)a.out + ((trow * a.H + h) * a.G + gv) * (long)DV + 4 * g4;
+#pragma unroll
+    for (int c = 0; c < VT; ++c) *reinterpret_cast<f32x4*>(o + 16 * c) = acc[c] * mul;
+    return;
   }
   T* o = (T*)a.out + (trow * a.H + h) * (long)DV + 4 * g4;
 #pragma unroll
@@ -1069,7 +1098,7 @@ VDAMD_API int vdamd_conv_norm_cache(const void* x, long x_stride, const void* co
 VDAMD_API int vdamd_short_conv_act(void* out, long out_stride, const void* x, long x_stride, const void* conv_w,
                                    void* state, const int* slots, const int* qsl, const int* seq_lens,
                                    const int* token_seq, const int* positions, int T, int B, int C, int taps, int silu,
-                                   int update_multi, int dt, hipStream_t stream) {
+                                   int update_multi, const float* bias, int residual, int dt, hipStream_t stream) {
   if (T <= 0) return 0;
   if (taps < 1 || taps > CONV_MAX_TAPS || C <= 0) return 1;
   const int R = taps - 1;
@@ -1082,14 +1111,14 @@ VDAMD_API int vdamd_short_conv_act(void* out, long out_stride, const void* x, lo
       if (vec) {
         hipLaunchKernelGGL((short_conv_act_kernel<TT, true>), dim3(T, (C / 8 + 255) / 256), dim3(256), 0, stream,
                            (TT*)out, out_stride, (const TT*)x, x_stride, (const TT*)conv_w, (TT*)state, slots, qsl,
-                           seq_lens, token_seq, positions, C, taps, silu);
+                           seq_lens, token_seq, positions, C, taps, silu, bias, residual);
         done = true;
       }
     }
     if (!done)
       hipLaunchKernelGGL((short_conv_act_kernel<TT, false>), dim3(T, (C + 255) / 256), dim3(256), 0, stream, (TT*)out,
                          out_stride, (const TT*)x, x_stride, (const TT*)conv_w, (TT*)state, slots, qsl, seq_lens,
-                         token_seq, positions, C, taps, silu);
+                         token_seq, positions, C, taps, silu, bias, residual);
     if (update_multi && R > 0)
       hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3((C + 255) / 256, B), dim3(256), 0, stream,
                          (const TT*)x, x_stride, (TT*)state, slots, qsl, C, R);
@@ -1124,13 +1153,14 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
                                           const void* gate, long gate_stride, void* out, int T, int B, int H, int G,
                                           int D, int Dv, int block_size, int window, int keep_first,
                                           int max_query_len, float scale, float softcap, int use_mfma, int chunk,
-                                          int dt, hipStream_t stream) {
+                                          int cross, int dt, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H % G || D <= 0 || Dv <= 0 || Dv > 64 * ATTN_V_PER_LANE || block_size <= 0 || block_size % 8 ||
-      (bias_scale && !bias_rate) || chunk < 0)
+      (bias_scale && !bias_rate) || chunk < 0 || (cross && (gate || sinks)))
     return 1;
   AttnArgs a{q, k_cache, v_cache, block_table, bt_stride, token_seq, positions, bias_scale, bias_rate, sinks, gate,
-             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap, chunk};
+             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap, chunk, cross ? 1 : 0};
+  const int gy = cross ? G * G : G;               // key heads, or (key head, value head) pairs
   const int qpg = H / G;
   const int dtiles = D / 32, vtiles = Dv / 16;
   if (use_mfma && dt == DT_BF16 && qsl && seq_lens && B > 0 && max_query_len > 0 && D % 32 == 0 && Dv % 16 == 0 &&
@@ -1143,7 +1173,7 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
     if (max_query_len <= tpw) { tw = 1; kw = 4; }          // few rows, many keys: the waves share the keys
     const int gx = (max_query_len + tw * tpw - 1) / (tw * tpw);
     const size_t lds = kw > 1 ? (size_t)tw * kw * 64 * (2 + 4 * vtiles) * sizeof(float) : 0;
-    const dim3 grid(gx, G * hchunks, B), block(64 * tw * kw);
+    const dim3 grid(gx, gy * hchunks, B), block(64 * tw * kw);
     switch (dtiles) {
       case 1: return launch_mfma<1>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
       case 2: return launch_mfma<2>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
@@ -1159,8 +1189,8 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
   return by_dtype(dt, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
     if (vec)
-      hipLaunchKernelGGL((window_bias_attention_kernel<TT, true>), dim3(T, G, chunks), dim3(64 * waves), lds, stream, a);
+      hipLaunchKernelGGL((window_bias_attention_kernel<TT, true>), dim3(T, gy, chunks), dim3(64 * waves), lds, stream, a);
     else
-      hipLaunchKernelGGL((window_bias_attention_kernel<TT, false>), dim3(T, G, chunks), dim3(64 * waves), lds, stream, a);
+      hipLaunchKernelGGL((window_bias_attention_kernel<TT, false>), dim3(T, gy, chunks), dim3(64 * waves), lds, stream, a);
   });
 }

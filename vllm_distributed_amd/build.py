@@ -31,7 +31,7 @@ HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffast-mat
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # sources whose fp32 arithmetic is part of a model's definition (norms, scores, softmax in 32-bit): IEEE division,
 # square roots and library exp / log / tanh instead of the fast-math forms
-EXACT_MATH_SOURCES = {"seq_mix.hip", "linear_latent.hip", "residual_rms.hip", "delta_rule.hip"}
+EXACT_MATH_SOURCES = {"seq_mix.hip", "linear_latent.hip", "residual_rms.hip", "delta_rule.hip", "state_space.hip"}
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-DNDEBUG"]
 
 

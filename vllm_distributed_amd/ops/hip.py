@@ -69,8 +69,12 @@ def load() -> ctypes.CDLL:
         "vdamd_scalar_norm_residual": [P, P, P, P, P, F, I, I, L, I, I, P],
         "vdamd_poly_norm": [P, P, P, F, I, I, L, I, P],
         "vdamd_conv_norm_cache": [P, L] + [P] * 16 + [I] * 8 + [F, I, P, I, I, P],
-        "vdamd_short_conv_act": [P, L, P, L, P, P, P, P, P, P, P] + [I] * 7 + [P],
-        "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, P, P, L, P] + [I] * 10 + [F, F, I, I, I, P],
+        "vdamd_short_conv_act": [P, L, P, L, P, P, P, P, P, P, P] + [I] * 6 + [P, I, I, P],
+        "vdamd_window_bias_attention": [P, P, P, P, L, P, P, P, P, P, P, P, P, L, P] + [I] * 10 + [F, F, I, I, I, I, P],
+        "vdamd_selective_scan": [P, P, L, P, L, P, P, P, P, P, P, P] + [I] * 7 + [P],
+        "vdamd_act_gate_group_norm": [P, P, P, L, P, F, I, I, I, I, P],
+        "vdamd_joint_norm_cache": [P, P, L, P, P, F, P, F, I, P, P, P] + [I] * 6 + [P],
+        "vdamd_mix_heads": [P, P, P, I, I, I, I, I, P],
         "vdamd_residual_rms": [P, L, P, L, P, L, P, L, P, L, P, P, F, F, I, I, I, I, I, I, P],
         "vdamd_gelu_mul_rows": [P, P, L, P, L, P, I, I, I, I, I, P],
         "vdamd_sigmoid_mul": [P, L, P, L, P, L, F, I, I, I, P],
@@ -1354,7 +1358,8 @@ def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, tok
 
 def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq_lens, token_seq, positions,
                           scale: float, softcap: float, window: int, keep_first: int, bias_scale, bias_rate, sinks,
-                          gate, max_query_len: int = 0, out=None, chunk: int = 0):
+                          gate, max_query_len: int = 0, out=None, chunk: int = 0, crossed: bool = False):
+    """``crossed``: every query head's weights on every value head, fp32 ``[T, H, Hkv, Dv]``."""
     t, h, d = q.shape
     g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     b = seq_lens.shape[0]
@@ -1369,9 +1374,11 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
     if gate is not None:
         assert gate.shape == (t, h) and gate.stride(1) == 1 and gate.dtype == q.dtype
         gate_stride = gate.stride(0)
+    out_shape, out_dtype = ((t, h, g, dv), torch.float32) if crossed else ((t, h, dv), q.dtype)
+    assert not crossed or (gate is None and sinks is None)
     if out is None:
-        out = torch.empty((t, h, dv), dtype=q.dtype, device=q.device)
-    assert out.shape == (t, h, dv) and out.dtype == q.dtype and out.is_contiguous()
+        out = torch.empty(out_shape, dtype=out_dtype, device=q.device)
+    assert out.shape == out_shape and out.dtype == out_dtype and out.is_contiguous()
     _check(_LIB.vdamd_window_bias_attention(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.stride(0),
         _ptr(_i32(token_seq, "token_seq")), _i32(positions, "positions").data_ptr(),
@@ -1379,7 +1386,7 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
         _ptr(_f32_vec(bias_scale, h, "bias_scale")), _ptr(_f32_vec(bias_rate, h, "bias_rate")),
         _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride, out.data_ptr(), t, b, h, g, d, dv, bs,
         int(window), int(keep_first), int(max_query_len) if max_query_len else t, float(scale), float(softcap),
-        1 if WINDOW_ATTENTION_MFMA else 0, int(chunk), _dt(q), _stream()), "window_bias_attention")
+        1 if WINDOW_ATTENTION_MFMA else 0, int(chunk), 1 if crossed else 0, _dt(q), _stream()), "window_bias_attention")
     return out
 
 
@@ -1631,7 +1638,7 @@ def gelu(x: torch.Tensor, tanh: bool) -> torch.Tensor:
 
 
 def short_conv_act(x, channels: int, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions,
-                   silu: bool, has_prefill: bool = True) -> torch.Tensor:
+                   silu: bool, has_prefill: bool = True, bias=None, residual: bool = False) -> torch.Tensor:
     t = _rows2d(x, "x").shape[0]
     c, taps = int(channels), conv_weight.shape[0]
     r = max(taps - 1, 1)
@@ -1649,8 +1656,8 @@ def short_conv_act(x, channels: int, conv_weight, state, slots, query_start_loc,
         out.data_ptr(), c, x.data_ptr(), x.stride(0), conv_weight.data_ptr(), state.data_ptr(),
         _i32(slots, "slots").data_ptr(), _i32(query_start_loc, "query_start_loc").data_ptr(),
         _i32(seq_lens, "seq_lens").data_ptr(), _ptr(_i32(token_seq, "token_seq")),
-        _i32(positions, "positions").data_ptr(), t, b, c, taps, 1 if silu else 0, 1 if has_prefill else 0, _dt(x),
-        _stream()), "short_conv_act")
+        _i32(positions, "positions").data_ptr(), t, b, c, taps, 1 if silu else 0, 1 if has_prefill else 0,
+        _ptr(_f32_vec(bias, c, "bias")), 1 if residual else 0, _dt(x), _stream()), "short_conv_act")
     return out
 
 
@@ -1682,4 +1689,71 @@ def gated_delta_rule(x, num_heads: int, num_qk_heads: int, dim: int, vdim: int, 
         bsig.data_ptr(), state.data_ptr(), _i32(slots, "slots").data_ptr(),
         _i32(query_start_loc, "query_start_loc").data_ptr(), _i32(seq_lens, "seq_lens").data_ptr(), b, h, g, dim, vdim,
         int(max_query_len), int(parts), _dt(x), _stream()), "gated_delta_rule")
+    return out
+
+
+# ------------------------------------------------ selective state-space scan, gate in front of a grouped norm,
+# ------------------------------------------------ q / k normed over all heads with values = keys, mixed head weights
+def selective_scan(x, dt, num_heads: int, groups: int, vdim: int, n_state: int, a_log, dt_bias, d_skip, state, slots,
+                   query_start_loc, seq_lens, max_query_len: int = 0) -> torch.Tensor:
+    """``max_query_len`` (0: unknown) only helps the kernel choose its launch."""
+    t = _rows2d(x, "x").shape[0]
+    h, g, n = int(num_heads), int(groups), int(n_state)
+    b = seq_lens.shape[0]
+    assert h % g == 0 and 0 < n <= 256 and x.shape[1] >= h * vdim + 2 * g * n
+    assert _rows2d(dt, "dt").shape[0] >= t and dt.shape[1] >= h and dt.dtype == x.dtype
+    assert state is not None and state.dtype == torch.float32 and state.is_contiguous()
+    assert tuple(state.shape[1:]) == (h, n, vdim), (tuple(state.shape), (h, n, vdim))
+    assert slots.shape[0] == b and query_start_loc.shape[0] >= b + 1
+    out = torch.empty((t, h * vdim), dtype=torch.float32, device=x.device)
+    _check(_LIB.vdamd_selective_scan(
+        out.data_ptr(), x.data_ptr(), x.stride(0), dt.data_ptr(), dt.stride(0), _f32_vec(a_log, h, "a_log").data_ptr(),
+        _f32_vec(dt_bias, h, "dt_bias").data_ptr(), _ptr(_f32_vec(d_skip, h, "d_skip")), state.data_ptr(),
+        _i32(slots, "slots").data_ptr(), _i32(query_start_loc, "query_start_loc").data_ptr(),
+        _i32(seq_lens, "seq_lens").data_ptr(), b, h, g, n, int(vdim), int(max_query_len), _dt(x), _stream()),
+        "selective_scan")
+    return out
+
+
+def act_gate_group_norm(y: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, group: int,
+                        out_dtype: torch.dtype) -> torch.Tensor:
+    t, n = y.shape
+    group = int(group) or n
+    assert y.dtype == torch.float32 and y.is_contiguous() and n % group == 0
+    assert _rows2d(gate, "gate").shape[0] >= t and gate.shape[1] >= n and gate.dtype == out_dtype
+    out = torch.empty((t, n), dtype=out_dtype, device=y.device)
+    _check(_LIB.vdamd_act_gate_group_norm(out.data_ptr(), y.data_ptr(), gate.data_ptr(), gate.stride(0),
+                                          _f32_vec(weight, n, "weight").data_ptr(), float(eps), t, n, group,
+                                          _dt(out), _stream()), "act_gate_group_norm")
+    return out
+
+
+def joint_norm_cache(x, num_heads: int, num_kv_heads: int, dim: int, q_norm, k_norm, eps: float, positions,
+                     temp_coef: float, temp_every: int, k_cache, v_cache, slot_mapping) -> torch.Tensor:
+    t = _rows2d(x, "x").shape[0]
+    h, g, d = int(num_heads), int(num_kv_heads), int(dim)
+    assert x.shape[1] >= (h + g) * d and positions.shape[0] >= t
+    bs = 0
+    if k_cache is not None:
+        bs = k_cache.shape[2]
+        assert k_cache.dtype == v_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
+        assert tuple(k_cache.shape[1:]) == (g, bs, d) and bs % 8 == 0
+        assert tuple(v_cache.shape) == (k_cache.shape[0], g, bs // 8, d, 8)
+        assert slot_mapping.shape[0] >= t
+    q = torch.empty((t, h, d), dtype=x.dtype, device=x.device)
+    _check(_LIB.vdamd_joint_norm_cache(
+        q.data_ptr(), x.data_ptr(), x.stride(0), _f32_vec(q_norm, h * d, "q_norm").data_ptr(),
+        _f32_vec(k_norm, g * d, "k_norm").data_ptr(), float(eps), _i32(positions, "positions").data_ptr(),
+        float(temp_coef), int(temp_every), _ptr(k_cache), _ptr(v_cache),
+        _ptr(_i32(slot_mapping, "slot_mapping") if k_cache is not None else None), t, h, g, d, int(bs), _dt(x),
+        _stream()), "joint_norm_cache")
+    return q
+
+
+def mix_heads(o: torch.Tensor, talk: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    t, h, g, dv = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous() and h % g == 0
+    out = torch.empty((t, h * dv), dtype=out_dtype, device=o.device)
+    _check(_LIB.vdamd_mix_heads(out.data_ptr(), o.data_ptr(), _f32_vec(talk, h * h, "talk").data_ptr(), t, h, g, dv,
+                                _dt(out), _stream()), "mix_heads")
     return out
