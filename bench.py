@@ -139,10 +139,10 @@ def _parse():
     ap.add_argument("--alt-parallelism", type=str, default="pp",
                     help="second layout measured in a child process after the headline when N > 1 ('none' = skip)")
     ap.add_argument("--alt-timeout", type=float, default=900.0)
-    ap.add_argument("--family-compare", type=str, default=None, choices=[None, "tavulix", "kabapel", "gosizen"],
+    ap.add_argument("--family-compare", type=str, default=None, choices=[None, "tavulix", "kabapel", "gosizen", "nalasun"],
                     help="instead of the headline: prefill and decode throughput of this model family at a few layer "
                          "sizes beside the closest existing family at equal size (Tavulix: Gemma-2; Kabapel: "
-                         "DeepSeek-V2; Gosizen: Kabapel), random weights, one GPU")
+                         "DeepSeek-V2; Gosizen: Kabapel; Nalasun: Gosizen), random weights, one GPU")
     ap.add_argument("--compare-sizes", type=str, default="small,medium",
                     help="with --family-compare: which of small / medium / large to run")
     ap.add_argument("--compare-only", type=str, default=None,
@@ -299,6 +299,29 @@ def _gosizen_models(z: dict) -> dict:
     return {"gosizen": ("gosizen-tiny", gos), "kabapel": _kabapel_models(z)["kabapel"]}
 
 
+def _nalasun_models(z: dict) -> dict:
+    """The same layer sizes as a Nalasun config (attention with keys as values and mixed head weights, the gated delta
+    rule, a state-space recurrence and attention again, in turn; every layer behind an input convolution and with an
+    expert block plus shared expert) and as a Gosizen config (attention over convolved keys beside the gated delta
+    rule, latent attention, expert blocks around an fp32 residual stream: the closest family the framework has)."""
+    vocab = 32000
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"] + z["identity"], "top": z["top"], "scale": 2.5}, "shared": {"ff": z["shared"]}}
+    kv = max(z["heads"] // 4, 1)
+    groups = max(z["heads"] // 8, 1)
+    mixers = [("attention", {"heads": z["heads"], "kv_heads": kv, "dim": z["nope"], "vdim": z["nope"],
+                             "scale": z["nope"] ** -0.5, "q_temp": {"coef": 0.1, "every": 256}}),
+              ("channel_delta", {"heads": z["heads"], "kv_heads": z["heads"], "dim": z["nope"], "vdim": z["vdim"], "conv": 4,
+                                 "decay_rank": 64, "gate_rank": 64}),
+              ("mamba2", {"heads": z["heads"], "vdim": z["vdim"], "state": z["nope"], "groups": groups,
+                          "norm_groups": groups, "conv": 4})]
+    order = [0, 1, 2, 0]
+    layers = [{"type": mixers[order[i % 4]][0], "mixer": mixers[order[i % 4]][1], "mlp": moe} for i in range(z["layers"])]
+    nal = {"architecture": "Nalasun", "vocab": vocab, "width": z["width"], "max_positions": 8192, "norm": {"eps": 1e-5},
+           "canon": {"taps": 4}, "layers": layers}
+    return {"nalasun": ("nalasun-tiny", nal), "gosizen": _gosizen_models(z)["gosizen"]}
+
+
 def run_family_compare(args) -> None:
     """Prefill throughput (``prompts`` prompts of ``prompt`` tokens, one generated token each) and decode
     throughput (``batch`` sequences, 64 further tokens each; the prefill time measured the same way is taken off)
@@ -308,11 +331,11 @@ def run_family_compare(args) -> None:
     from vllm_distributed_amd import LLM, SamplingParams
     os.environ.setdefault("VLLM_LOGGING_LEVEL", "WARNING")
     rows = []
-    kabapel = args.family_compare in ("kabapel", "gosizen")
+    kabapel = args.family_compare in ("kabapel", "gosizen", "nalasun")
     for size in [s for s in args.compare_sizes.split(",") if s]:
         z = (KABAPEL_SIZES if kabapel else COMPARE_SIZES)[size]
-        models = (_gosizen_models(z) if args.family_compare == "gosizen" else _kabapel_models(z)) if kabapel \
-            else _compare_models(z)
+        by_family = {"gosizen": _gosizen_models, "nalasun": _nalasun_models, "kabapel": _kabapel_models}
+        models = by_family[args.family_compare](z) if kabapel else _compare_models(z)
         for family, (base, over) in models.items():
             if args.compare_only and family != args.compare_only:
                 continue

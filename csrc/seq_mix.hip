@@ -581,8 +581,11 @@ struct AttnArgs {
   int T, H, G, D, Dv, block_size, window, keep_first;
   float scale, softcap;
   int chunk;                        // > 0: a query sees only the keys of its own block of `chunk` positions
-  int cross;                        // 1: every query head's weights are applied to the values of EVERY key / value head,
-                                    // out is fp32 [T, H, G, Dv] (blockIdx.y then counts (key head, value head) pairs)
+  int cross;                        // > 0: every query head's weights are applied to the values of EVERY key / value head,
+                                    // out is fp32 [T, H, G, Dv] (blockIdx.y then counts (key head, value head(s)) pairs)
+  int xcd_seqs;                     // > 0 (= sequences; grid.x == 1, grid.z padded to a multiple of 8): the workgroups of
+                                    // one sequence are dealt to ONE of the chip's 8 dies (workgroups go to the dies in
+                                    // turn by their linear number), so that what they all read is shared in its L2
 };
 
 template <typename T, bool VEC> struct RowDot;
@@ -740,8 +743,10 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
 // interleave so that a lane ends up with 8 consecutive keys of ITS query row), cap / bias / mask / online softmax in
 // fp32 per lane, O^T += V^T P^T with P split into bf16 high and low parts.  Everything a query row needs (max, sum,
 // rescale factor, its O^T column) lives in the lanes with l % 16 == row.  With `kw` > 1 the block's waves take the
-// key steps in turn for the same rows and are merged through LDS (decode: few rows, many keys).
-template <int DT, int VT>
+// key steps in turn for the same rows and are merged through LDS (decode: few rows, many keys).  CG > 1 (crossed
+// value heads only): the step's weights are applied to CG value heads in turn, each with accumulators of its own, so
+// the scores and the softmax are computed once for all of them.
+template <int DT, int VT, int CG>
 __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArgs a, const int* __restrict__ qsl,
                                                                          const int* __restrict__ seq_lens, int hp,
                                                                          int tpw, int kw) {
@@ -752,12 +757,20 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   constexpr float LOG2E = 1.4426950408889634f;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int r16 = lane & 15, g4 = lane >> 4;
-  const int s = blockIdx.z;
+  int s = blockIdx.z, by = blockIdx.y;
+  if (a.xcd_seqs > 0) {
+    const int linear = blockIdx.y + gridDim.y * blockIdx.z;
+    const int die = linear & 7, slot = linear >> 3;
+    s = die + 8 * (slot / (int)gridDim.y);
+    by = slot % (int)gridDim.y;
+    if (s >= a.xcd_seqs) return;                  // (the whole workgroup)
+  }
   const int qpg = a.H / a.G;
   const int hchunks = (qpg + hp - 1) / hp;
-  const int gy = blockIdx.y / hchunks, hc = blockIdx.y % hchunks;
-  const int g = a.cross ? gy / a.G : gy;          // key head
-  const int gv = a.cross ? gy % a.G : g;          // value head
+  const int gy = by / hchunks, hc = by % hchunks;
+  const int vchunks = a.cross ? (a.G + CG - 1) / CG : 1;
+  const int g = a.cross ? gy / vchunks : gy;                  // key head
+  const int gv0 = a.cross ? (gy % vchunks) * CG : g;          // first value head (the only one unless crossed)
   const int tw = nwaves / kw;                     // waves over tokens
   const int wt = wave / kw, wk = wave % kw;
   const int q0 = qsl[s], n_tok = qsl[s + 1] - q0;
@@ -808,9 +821,11 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     if (bs_shift >= 0) { bi = key >> bs_shift; off = key & (bs - 1); }
     else { bi = key / bs; off = key - bi * bs; }
   };
-  f32x4 acc[VT];
+  f32x4 acc[CG][VT];
 #pragma unroll
-  for (int c = 0; c < VT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int cc = 0; cc < CG; ++cc)
+#pragma unroll
+    for (int c = 0; c < VT; ++c) acc[cc][c] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   int lo_row = a.window > 0 ? pos - a.window + 1 : 0;
   if (a.chunk > 0) lo_row = max(lo_row, pos - pos % a.chunk);
@@ -845,7 +860,8 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     const int vkey = min(base + 8 * g4, p_last) & ~7;
     split(vkey, bi_v, off_v);
     const long blk_v = bt[bi_v];
-    const T* vp = vc + (((blk_v * a.G + gv) * bs8 + (off_v >> 3)) * (long)DV + r16) * 8;
+    const long vhead = (long)bs8 * DV * 8;         // from a value head's fragments to the next head's
+    const T* vp = vc + (((blk_v * a.G + gv0) * bs8 + (off_v >> 3)) * (long)DV + r16) * 8;
     V8 vf[VT];
 #pragma unroll
     for (int c = 0; c < VT; ++c) vf[c] = ld8<T>(vp + (long)c * 128);
@@ -893,42 +909,73 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     m = m_new;
     if (__any(alpha != 1.f)) {
 #pragma unroll
-      for (int c = 0; c < VT; ++c) acc[c] *= alpha;
+      for (int cc = 0; cc < CG; ++cc)
+#pragma unroll
+        for (int c = 0; c < VT; ++c) acc[cc][c] *= alpha;
     }
 #pragma unroll
-    for (int c = 0; c < VT; ++c) {
-      acc[c] = mfma16(vf[c], ph, acc[c]);
-      acc[c] = mfma16(vf[c], pl, acc[c]);
-    }
-  }
-  // ---- merge the key-split waves of a row set (wave wk == 0 of each set ends up with the result)
-  if (kw > 1) {
-    // per (token-wave, key-wave, lane): m, l, VT * 4 accumulators
-    const int per = 2 + 4 * VT;
-    float* mine = lds + ((long)(wt * kw + wk) * 64 + lane) * per;
-    if (wk > 0) {
-      mine[0] = m; mine[1] = l;
+    for (int cc = 0; cc < CG; ++cc) {
+      V8 vn[VT];
+      if (cc + 1 < CG) {                           // the next value head's fragments, in flight during this head's MFMAs
+        const T* vq = vp + (long)min(cc + 1, a.G - 1 - gv0) * vhead;
 #pragma unroll
-      for (int c = 0; c < VT; ++c) { mine[2 + 4 * c] = acc[c][0]; mine[3 + 4 * c] = acc[c][1]; mine[4 + 4 * c] = acc[c][2]; mine[5 + 4 * c] = acc[c][3]; }
-    }
-    __syncthreads();
-    if (wk > 0) return;
-    for (int o = 1; o < kw; ++o) {
-      const float* th = lds + ((long)(wt * kw + o) * 64 + lane) * per;
-      const float m_o = th[0], l_o = th[1];
-      const float m_new = fmaxf(m, m_o);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float fa = fast_exp2(m - m_use), fb = fast_exp2(m_o - m_use);
-      l = l * fa + l_o * fb;
-      m = m_new;
+        for (int c = 0; c < VT; ++c) vn[c] = ld8<T>(vq + (long)c * 128);
+      }
 #pragma unroll
       for (int c = 0; c < VT; ++c) {
-        acc[c][0] = acc[c][0] * fa + th[2 + 4 * c] * fb;
-        acc[c][1] = acc[c][1] * fa + th[3 + 4 * c] * fb;
-        acc[c][2] = acc[c][2] * fa + th[4 + 4 * c] * fb;
-        acc[c][3] = acc[c][3] * fa + th[5 + 4 * c] * fb;
+        acc[cc][c] = mfma16(vf[c], ph, acc[cc][c]);
+        acc[cc][c] = mfma16(vf[c], pl, acc[cc][c]);
+      }
+      if (cc + 1 < CG) {
+#pragma unroll
+        for (int c = 0; c < VT; ++c) vf[c] = vn[c];
       }
     }
+  }
+  // ---- merge the key-split waves of a row set (wave wk == 0 of each set ends up with the result): every wave
+  // brings its sums to the common maximum, then wave 0 adds them up, one value head at a time
+  if (kw > 1) {
+    float* ml = lds;                                                    // [tw * kw * 64][2]
+    float* buf = lds + (long)tw * kw * 64 * 2;                          // [tw * kw * 64][4 * VT]
+    float* mine = ml + ((long)(wt * kw + wk) * 64 + lane) * 2;
+    mine[0] = m; mine[1] = l;
+    __syncthreads();
+    float m_all = m;
+    for (int o = 0; o < kw; ++o) m_all = fmaxf(m_all, ml[((long)(wt * kw + o) * 64 + lane) * 2]);
+    const float m_use = m_all == -INFINITY ? 0.f : m_all;
+    float l_all = 0.f;
+    for (int o = 0; o < kw; ++o) {
+      const float* th = ml + ((long)(wt * kw + o) * 64 + lane) * 2;
+      l_all += th[1] * fast_exp2(th[0] - m_use);
+    }
+    const float fs = fast_exp2(m - m_use);
+    m = m_all; l = l_all;
+#pragma unroll
+    for (int cc = 0; cc < CG; ++cc) {
+      float* pa = buf + ((long)(wt * kw + wk) * 64 + lane) * (4 * VT);
+      if (wk > 0) {
+#pragma unroll
+        for (int c = 0; c < VT; ++c) {
+          pa[4 * c] = acc[cc][c][0] * fs; pa[4 * c + 1] = acc[cc][c][1] * fs;
+          pa[4 * c + 2] = acc[cc][c][2] * fs; pa[4 * c + 3] = acc[cc][c][3] * fs;
+        }
+      }
+      __syncthreads();
+      if (wk == 0) {
+#pragma unroll
+        for (int c = 0; c < VT; ++c) acc[cc][c] *= fs;
+        for (int o = 1; o < kw; ++o) {
+          const float* th = buf + ((long)(wt * kw + o) * 64 + lane) * (4 * VT);
+#pragma unroll
+          for (int c = 0; c < VT; ++c) {
+            acc[cc][c][0] += th[4 * c]; acc[cc][c][1] += th[4 * c + 1];
+            acc[cc][c][2] += th[4 * c + 2]; acc[cc][c][3] += th[4 * c + 3];
+          }
+        }
+      }
+      if (cc + 1 < CG) __syncthreads();
+    }
+    if (wk > 0) return;
   }
   if (!row_ok) return;
   if (a.sinks) {
@@ -937,17 +984,21 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     const float fa = fast_exp2(m - m_f);
     l = l * fa + fast_exp2(sk - m_f);
 #pragma unroll
-    for (int c = 0; c < VT; ++c) acc[c] *= fa;
+    for (int c = 0; c < VT; ++c) acc[0][c] *= fa;
   }
   float mul = 1.0f / l;
   if (a.gate) {
-    const float gv = (float)((const T*)a.gate)[trow * a.gate_stride + h];
-    mul *= 1.0f / (1.0f + expf(-gv));
+    const float gate_v = (float)((const T*)a.gate)[trow * a.gate_stride + h];
+    mul *= 1.0f / (1.0f + expf(-gate_v));
   }
   if (a.cross) {
-    float* o = (float*)a.out + ((trow * a.H + h) * a.G + gv) * (long)DV + 4 * g4;
 #pragma unroll
-    for (int c = 0; c < VT; ++c) *reinterpret_cast<f32x4*>(o + 16 * c) = acc[c] * mul;
+    for (int cc = 0; cc < CG; ++cc) {
+      if (gv0 + cc >= a.G) break;
+      float* o = (float*)a.out + ((trow * a.H + h) * a.G + gv0 + cc) * (long)DV + 4 * g4;
+#pragma unroll
+      for (int c = 0; c < VT; ++c) *reinterpret_cast<f32x4*>(o + 16 * c) = acc[cc][c] * mul;
+    }
     return;
   }
   T* o = (T*)a.out + (trow * a.H + h) * (long)DV + 4 * g4;
@@ -955,7 +1006,7 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   for (int c = 0; c < VT; ++c) {
     bf16x4 ov;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ov[i] = (T)(acc[c][i] * mul);
+    for (int i = 0; i < 4; ++i) ov[i] = (T)(acc[0][c][i] * mul);
     *reinterpret_cast<bf16x4*>(o + 16 * c) = ov;
   }
 }
@@ -1127,25 +1178,38 @@ VDAMD_API int vdamd_short_conv_act(void* out, long out_stride, const void* x, lo
 
 namespace {
 
-template <int DT> int launch_mfma(int vt, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const AttnArgs& a,
-                                  const int* qsl, const int* seq_lens, int hp, int tpw, int kw) {
+template <int DT, int CG> int launch_mfma(int vt, dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                                          const AttnArgs& a, const int* qsl, const int* seq_lens, int hp, int tpw,
+                                          int kw) {
   switch (vt) {
-#define VDAMD_CASE(VT_)                                                                                         \
-  case VT_:                                                                                                     \
-    hipLaunchKernelGGL((window_bias_attention_mfma_kernel<DT, VT_>), grid, block, lds, stream, a, qsl, seq_lens, \
-                       hp, tpw, kw);                                                                            \
-    return 0;
+#define VDAMD_CASE(VT_)                                                                                              \
+  case VT_:                                                                                                          \
+    if constexpr (CG * VT_ <= 32) {                                                                                  \
+      hipLaunchKernelGGL((window_bias_attention_mfma_kernel<DT, VT_, CG>), grid, block, lds, stream, a, qsl,         \
+                         seq_lens, hp, tpw, kw);                                                                     \
+      return 0;                                                                                                      \
+    }                                                                                                                \
+    return 1;
     VDAMD_CASE(1) VDAMD_CASE(2) VDAMD_CASE(4) VDAMD_CASE(8)
 #undef VDAMD_CASE
   }
   return 1;
 }
 
+// value heads a workgroup of the crossed form takes: as many as share one computation of the scores without the
+// accumulators (CG * Dv / 16 vectors of four) outgrowing the register file
+int cross_group(int G, int vtiles) {
+  int cg = G >= 3 ? 4 : (G == 2 ? 2 : 1);
+  while (cg > 1 && cg * vtiles > 32) cg >>= 1;
+  return cg;
+}
+
 }  // namespace
 
 // q [T, H, D]; sequence b owns rows qsl[b] .. qsl[b + 1], the last positions of its seq_lens[b] tokens
 // (token_seq / positions say the same per row, for the kernel that walks rows).  use_mfma: 0 never, 1 when the
-// shape allows (bf16, D a multiple of 32 up to 256, Dv in {16, 32, 64, 128}).
+// shape allows (bf16, D a multiple of 32 up to 256, Dv in {16, 32, 64, 128}).  cross: 0, or the most value heads
+// (1, 2 or 4) that may share one computation of the scores in the crossed form.
 VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, const void* v_cache,
                                           const int* block_table, long bt_stride, const int* token_seq,
                                           const int* positions, const int* qsl, const int* seq_lens,
@@ -1159,7 +1223,7 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
       (bias_scale && !bias_rate) || chunk < 0 || (cross && (gate || sinks)))
     return 1;
   AttnArgs a{q, k_cache, v_cache, block_table, bt_stride, token_seq, positions, bias_scale, bias_rate, sinks, gate,
-             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap, chunk, cross ? 1 : 0};
+             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap, chunk, cross ? 1 : 0, 0};
   const int gy = cross ? G * G : G;               // key heads, or (key head, value head) pairs
   const int qpg = H / G;
   const int dtiles = D / 32, vtiles = Dv / 16;
@@ -1173,13 +1237,20 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
     if (max_query_len <= tpw) { tw = 1; kw = 4; }          // few rows, many keys: the waves share the keys
     const int gx = (max_query_len + tw * tpw - 1) / (tw * tpw);
     const size_t lds = kw > 1 ? (size_t)tw * kw * 64 * (2 + 4 * vtiles) * sizeof(float) : 0;
-    const dim3 grid(gx, gy * hchunks, B), block(64 * tw * kw);
-    switch (dtiles) {
-      case 1: return launch_mfma<1>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
-      case 2: return launch_mfma<2>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
-      case 4: return launch_mfma<4>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
-      case 8: return launch_mfma<8>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
+    const int cg = cross ? (cross_group(G, vtiles) < cross ? cross_group(G, vtiles) : cross) : 1;
+    const int pairs = cross ? G * ((G + cg - 1) / cg) : G;      // (key head, group of value heads)
+    dim3 grid(gx, pairs * hchunks, B), block(64 * tw * kw);
+    if (cross && gx == 1 && pairs * hchunks > 1) {          // decoded rows: a sequence's workgroups on one die
+      a.xcd_seqs = B;
+      grid.z = (B + 7) / 8 * 8;
     }
+#define VDAMD_DT(DT_)                                                                                          \
+  case DT_:                                                                                                    \
+    if (cg == 4) return launch_mfma<DT_, 4>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);  \
+    if (cg == 2) return launch_mfma<DT_, 2>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);  \
+    return launch_mfma<DT_, 1>(vtiles, grid, block, lds, stream, a, qsl, seq_lens, hp, tpw, kw);
+    switch (dtiles) { VDAMD_DT(1) VDAMD_DT(2) VDAMD_DT(4) VDAMD_DT(8) }
+#undef VDAMD_DT
   }
   const int waves = qpg < ATTN_MAX_WAVES ? qpg : ATTN_MAX_WAVES;
   const int chunks = (qpg + waves - 1) / waves;

@@ -13,6 +13,7 @@
 //                         factor 1 + coef * ln(floor((p + 1) / every) + 1), normed k into the key rows, the projected
 //                         k into the values (eight keys side by side per channel)
 //   mix_heads             out[t, h] = sum_g talk[h, g] * o[t, g, kv(h)] over fp32 [T, H, G, Dv]
+// The 16-bit forms of the two norm kernels give a lane 8 neighbouring columns (16-byte accesses).
 #include "common.h"
 #include <math.h>
 #include <type_traits>
@@ -170,6 +171,51 @@ __global__ __launch_bounds__(256) void act_gate_group_norm_kernel(T* __restrict_
   }
 }
 
+// the same for 16-bit gates and results with 8 columns per lane (16-byte accesses); a lane keeps up to P portions of
+// 8 gated values in registers between the sum of squares and the result, so a group of up to 8 * P * blockDim columns
+// is read once
+template <typename T, int P>
+__global__ __launch_bounds__(256) void act_gate_group_norm_vec_kernel(T* __restrict__ out, const float* __restrict__ y,
+                                                                      const T* __restrict__ gate, long gate_stride,
+                                                                      const float* __restrict__ w, float eps, int N,
+                                                                      int group) {
+  using V8 = typename Vec8<T>::type;
+  __shared__ float red[17];
+  const long t = blockIdx.x;
+  const int c0 = blockIdx.y * group;
+  const float* yr = y + t * N + c0;
+  const T* gr = gate + t * gate_stride + c0;
+  float z[P][8];
+  float sq = 0.f;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    const int i = (p * blockDim.x + threadIdx.x) * 8;
+    if (i < group) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(yr + i), b = *reinterpret_cast<const f32x4*>(yr + i + 4);
+      const V8 gv = ld8<T>(gr + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float gf = (float)gv[e];
+        z[p][e] = (e < 4 ? a[e & 3] : b[e & 3]) * (gf * sigmoid_f(gf));
+        sq += z[p][e] * z[p][e];
+      }
+    }
+  }
+  const float inv = 1.0f / sqrtf(block_sum(sq, red) / (float)group + eps);
+  T* o = out + t * N + c0;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    const int i = (p * blockDim.x + threadIdx.x) * 8;
+    if (i < group) {
+      const f32x4 wa = *reinterpret_cast<const f32x4*>(w + c0 + i), wb = *reinterpret_cast<const f32x4*>(w + c0 + i + 4);
+      V8 r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[e] = (T)(z[p][e] * inv * (e < 4 ? wa[e & 3] : wb[e & 3]));
+      st8<T>(o + i, r);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ q / k over all heads
 // grid (rows): x row = [q (H * D) | k (G * D)].
 template <typename T>
@@ -208,19 +254,89 @@ __global__ __launch_bounds__(256) void joint_norm_cache_kernel(T* __restrict__ q
   }
 }
 
+// the same for 16-bit types with 8 channels per lane (16-byte loads of the row, 16-byte stores of q and of the key
+// row; the values go eight 2-byte stores per lane, one per channel, into the key-grouped layout)
+template <typename T>
+__global__ __launch_bounds__(256) void joint_norm_cache_vec_kernel(T* __restrict__ q_out, const T* __restrict__ x,
+                                                                   long x_stride, const float* __restrict__ q_w,
+                                                                   const float* __restrict__ k_w, float eps,
+                                                                   const int* __restrict__ positions, float coef,
+                                                                   int every, T* __restrict__ k_cache,
+                                                                   T* __restrict__ v_cache,
+                                                                   const int* __restrict__ slot_mapping, int H, int G,
+                                                                   int D, int bs) {
+  using V8 = typename Vec8<T>::type;
+  __shared__ float red[17];
+  const long t = blockIdx.x;
+  const T* xr = x + t * x_stride;
+  const int qs = H * D, ks = G * D;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x * 8; i < qs + ks; i += blockDim.x * 8) {
+    const V8 v = ld8<T>(xr + i);
+    float a = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a += (float)v[e] * (float)v[e];
+    if (i < qs) sq += a; else sk += a;
+  }
+  sq = block_sum(sq, red);
+  sk = block_sum(sk, red);
+  float iq = 1.0f / sqrtf(sq / (float)qs + eps);
+  const float ik = 1.0f / sqrtf(sk / (float)ks + eps);
+  if (every > 0) iq *= 1.0f + coef * logf((float)((positions[t] + 1) / every) + 1.0f);
+  const int slot = k_cache != nullptr ? slot_mapping[t] : -1;
+  const long blk = slot >= 0 ? slot / bs : 0;
+  const int off = slot >= 0 ? slot % bs : 0;
+  T* qo = q_out + t * qs;
+  for (int i = threadIdx.x * 8; i < qs + ks; i += blockDim.x * 8) {
+    const V8 v = ld8<T>(xr + i);                                   // (the row is still in the cache)
+    const bool is_q = i < qs;
+    const float* wp = is_q ? q_w + i : k_w + (i - qs);
+    const f32x4 wa = *reinterpret_cast<const f32x4*>(wp), wb = *reinterpret_cast<const f32x4*>(wp + 4);
+    const float mul = is_q ? iq : ik;
+    V8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (T)((float)v[e] * mul * (e < 4 ? wa[e & 3] : wb[e & 3]));
+    if (is_q) {
+      st8<T>(qo + i, r);
+    } else if (slot >= 0) {
+      const int j = i - qs, g = j / D, d = j - g * D;              // (D % 8 == 0: the 8 channels share a head)
+      st8<T>(k_cache + ((blk * G + g) * bs + off) * (long)D + d, r);
+      T* vd = v_cache + (((blk * G + g) * (bs >> 3) + (off >> 3)) * (long)D + d) * 8 + (off & 7);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vd[e * 8] = v[e];
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ mixed head weights
-// grid (rows, heads): o fp32 [T, H, G, Dv]; head h sums talk[h, g] * o[t, g, h / (H / G)] over g.
+// grid (rows, key / value heads): o fp32 [T, H, G, Dv]; the heads h of key / value head c each sum
+// talk[h, g] * o[t, g, c] over g.  A lane owns a column d and four of those heads at a time, so every value of o is
+// read once per four heads.
 template <typename T>
 __global__ __launch_bounds__(256) void mix_heads_kernel(T* __restrict__ out, const float* __restrict__ o,
                                                         const float* __restrict__ talk, int H, int G, int Dv) {
   const long t = blockIdx.x;
-  const int h = blockIdx.y;
-  const int c = h / (H / G);
-  const float* tw = talk + (long)h * H;
+  const int c = blockIdx.y;
+  const int qpg = H / G;
+  const float* src = o + (t * H * G + c) * (long)Dv;               // + g * G * Dv + d
   for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
-    float acc = 0.f;
-    for (int g = 0; g < H; ++g) acc += tw[g] * o[((t * H + g) * G + c) * (long)Dv + d];
-    stf(out + (t * H + h) * (long)Dv + d, acc);
+    for (int h0 = 0; h0 < qpg; h0 += 4) {
+      const float* tw = talk + (long)(c * qpg + h0) * H;
+      const int nh = min(4, qpg - h0);
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      for (int g = 0; g < H; ++g) {
+        const float v = src[(long)g * G * Dv + d];
+        a0 += tw[g] * v;
+        if (nh > 1) a1 += tw[H + g] * v;
+        if (nh > 2) a2 += tw[2 * H + g] * v;
+        if (nh > 3) a3 += tw[3 * H + g] * v;
+      }
+      T* dst = out + (t * H + c * qpg + h0) * (long)Dv + d;
+      stf(dst, a0);
+      if (nh > 1) stf(dst + Dv, a1);
+      if (nh > 2) stf(dst + 2 * (long)Dv, a2);
+      if (nh > 3) stf(dst + 3 * (long)Dv, a3);
+    }
   }
 }
 
@@ -267,8 +383,28 @@ VDAMD_API int vdamd_act_gate_group_norm(void* out, const float* y, const void* g
   if (T <= 0) return 0;
   if (N <= 0 || group <= 0 || N % group) return 1;
   const int th = group >= 1024 ? 256 : (group >= 256 ? 128 : 64);
+  const bool vec = dtype != DT_F32 && group % 8 == 0 && gate_stride % 8 == 0 && ((uintptr_t)gate & 15) == 0 &&
+                   ((uintptr_t)out & 15) == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+                   group <= 8 * 4 * 256;
   const int rc = by_dtype(dtype, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
+    if constexpr (!std::is_same_v<TT, float>) {
+      if (vec) {
+        const int lanes = group / 8;                // a lane per 8 columns, up to 4 portions per lane
+        const int tv = lanes >= 256 ? 256 : (lanes >= 128 ? 128 : 64);
+        const dim3 grid(T, N / group);
+        if (lanes <= tv)
+          hipLaunchKernelGGL((act_gate_group_norm_vec_kernel<TT, 1>), grid, dim3(tv), 0, stream, (TT*)out, y,
+                             (const TT*)gate, gate_stride, w, eps, N, group);
+        else if (lanes <= 2 * tv)
+          hipLaunchKernelGGL((act_gate_group_norm_vec_kernel<TT, 2>), grid, dim3(tv), 0, stream, (TT*)out, y,
+                             (const TT*)gate, gate_stride, w, eps, N, group);
+        else
+          hipLaunchKernelGGL((act_gate_group_norm_vec_kernel<TT, 4>), grid, dim3(tv), 0, stream, (TT*)out, y,
+                             (const TT*)gate, gate_stride, w, eps, N, group);
+        return;
+      }
+    }
     hipLaunchKernelGGL((act_gate_group_norm_kernel<TT>), dim3(T, N / group), dim3(th), 0, stream, (TT*)out, y,
                        (const TT*)gate, gate_stride, w, eps, N, group);
   });
@@ -286,8 +422,20 @@ VDAMD_API int vdamd_joint_norm_cache(void* q_out, const void* x, long x_stride, 
   if (T <= 0) return 0;
   if (H <= 0 || G <= 0 || D <= 0 || every < 0) return 1;
   if (k_cache != nullptr && (v_cache == nullptr || slot_mapping == nullptr || bs <= 0 || bs % 8)) return 1;
+  const bool vec = dtype != DT_F32 && D % 8 == 0 && x_stride % 8 == 0 && ((uintptr_t)x & 15) == 0 &&
+                   ((uintptr_t)q_out & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && ((uintptr_t)q_w & 15) == 0 &&
+                   ((uintptr_t)k_w & 15) == 0;
   const int rc = by_dtype(dtype, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
+    if constexpr (!std::is_same_v<TT, float>) {
+      if (vec) {
+        const int lanes = (H + G) * D / 8;
+        hipLaunchKernelGGL((joint_norm_cache_vec_kernel<TT>), dim3(T), dim3(lanes >= 256 ? 256 : (lanes >= 128 ? 128 : 64)),
+                           0, stream, (TT*)q_out, (const TT*)x, x_stride, q_w, k_w, eps, positions, coef, every,
+                           (TT*)k_cache, (TT*)v_cache, slot_mapping, H, G, D, bs);
+        return;
+      }
+    }
     hipLaunchKernelGGL((joint_norm_cache_kernel<TT>), dim3(T), dim3(256), 0, stream, (TT*)q_out, (const TT*)x, x_stride,
                        q_w, k_w, eps, positions, coef, every, (TT*)k_cache, (TT*)v_cache, slot_mapping, H, G, D, bs);
   });
@@ -304,7 +452,7 @@ VDAMD_API int vdamd_mix_heads(void* out, const float* o, const float* talk, int 
   const int th = Dv >= 256 ? 256 : (Dv >= 128 ? 128 : 64);
   const int rc = by_dtype(dtype, [&](auto* tp) {
     using TT = std::remove_pointer_t<decltype(tp)>;
-    hipLaunchKernelGGL((mix_heads_kernel<TT>), dim3(T, H), dim3(th), 0, stream, (TT*)out, o, talk, H, G, Dv);
+    hipLaunchKernelGGL((mix_heads_kernel<TT>), dim3(T, G), dim3(th), 0, stream, (TT*)out, o, talk, H, G, Dv);
   });
   if (rc) return 1;
   HIP_LAUNCH_CHECK();

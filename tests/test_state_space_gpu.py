@@ -98,7 +98,8 @@ def test_selective_scan(dtype, h, groups, vdim, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("n,group", [(96, 32), (256, 256), (192, 64), (40, 5), (3072, 1536)])
+@pytest.mark.parametrize("n,group", [(96, 32), (256, 256), (192, 64), (40, 5), (3072, 1536), (4096, 4096), (8192, 8192),
+                                     (16400, 16400)])
 def test_act_gate_group_norm(dtype, n, group):
     hip = _hip()
     g = torch.Generator(device="cuda").manual_seed(n + group)
@@ -139,7 +140,8 @@ def test_joint_norm_cache(dtype, h, g, d, every):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("h,g,d", [(4, 2, 32), (6, 3, 64), (4, 4, 16), (2, 1, 128), (3, 3, 24), (8, 2, 64)])
+@pytest.mark.parametrize("h,g,d", [(4, 2, 32), (6, 3, 64), (4, 4, 16), (2, 1, 128), (3, 3, 24), (8, 2, 64), (8, 4, 128),
+                                   (16, 8, 32), (10, 2, 32), (5, 5, 64)])
 def test_crossed_attention_and_mixing(dtype, h, g, d):
     hip = _hip()
     gen = torch.Generator(device="cuda").manual_seed(h * 100 + d)

@@ -599,17 +599,24 @@ class BiasedTopKMoE(FusedMoE):
 
 class GatedMLP(nn.Module):
     """One feed-forward of the gated form ``down(silu(gate(x)) * up(x))``, gate and up as one fused projection; no
-    biases."""
+    biases.  The inner width is zero-padded to a multiple of 8 (the activation kernel's 16-byte accesses)."""
 
     def __init__(self, hidden: int, inter: int, dtype: torch.dtype):
         super().__init__()
-        self.inter = inter
-        self.w13 = nn.Parameter(torch.empty(2 * inter, hidden, dtype=dtype), requires_grad=False)
-        self.w2 = nn.Parameter(torch.empty(hidden, inter, dtype=dtype), requires_grad=False)
+        self.inter, self.i_pad = inter, (inter + 7) // 8 * 8
+        self.w13 = nn.Parameter(torch.zeros(2 * self.i_pad, hidden, dtype=dtype), requires_grad=False)
+        self.w2 = nn.Parameter(torch.zeros(hidden, self.i_pad, dtype=dtype), requires_grad=False)
         self.w13.weight_loader = self._load_w13
+        self.w2.weight_loader = self._load_w2
 
     def _load_w13(self, param: nn.Parameter, w: torch.Tensor, shard_id) -> None:
-        param.data.narrow(0, int(shard_id) * self.inter, self.inter).copy_(materialize(w))
+        dst = param.data.narrow(0, int(shard_id) * self.i_pad, self.i_pad)
+        dst.zero_()                          # (the padding included: the loader poisons fresh parameters)
+        dst[:self.inter].copy_(materialize(w))
+
+    def _load_w2(self, param: nn.Parameter, w: torch.Tensor, shard_id=None) -> None:
+        param.data.zero_()
+        param.data[:, :self.inter].copy_(materialize(w))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.linear(ops.silu_and_mul(ops.linear(x, self.w13)), self.w2)

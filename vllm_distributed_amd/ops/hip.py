@@ -1309,6 +1309,8 @@ CONV_MAX_TAPS = 16
 UNIT_MAX_WIDTH = 512
 # the matrix-core attention kernel where the shape allows it (tests switch it off to run the plain kernel in bf16)
 WINDOW_ATTENTION_MFMA = os.environ.get("VDAMD_WINDOW_ATTENTION_MFMA", "1") != "0"
+CROSS_GROUP_PROMPT = int(os.environ.get("VDAMD_CROSS_GROUP_PROMPT", "2"))
+CROSS_GROUP_DECODE = int(os.environ.get("VDAMD_CROSS_GROUP_DECODE", "2"))
 
 
 def conv_norm_cache(x, conv_weight, state, slots, query_start_loc, seq_lens, token_seq, positions, num_heads: int,
@@ -1375,6 +1377,9 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
         assert gate.shape == (t, h) and gate.stride(1) == 1 and gate.dtype == q.dtype
         gate_stride = gate.stride(0)
     out_shape, out_dtype = ((t, h, g, dv), torch.float32) if crossed else ((t, h, dv), q.dtype)
+    # value heads that share one computation of the scores (measured: with four, the accumulators of four heads
+    # leave a SIMD one resident wave, and both prompt portions and decoded rows run slower than with two)
+    cross = 0 if not crossed else (CROSS_GROUP_DECODE if max_query_len == 1 else CROSS_GROUP_PROMPT)
     assert not crossed or (gate is None and sinks is None)
     if out is None:
         out = torch.empty(out_shape, dtype=out_dtype, device=q.device)
@@ -1386,7 +1391,7 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
         _ptr(_f32_vec(bias_scale, h, "bias_scale")), _ptr(_f32_vec(bias_rate, h, "bias_rate")),
         _ptr(_f32_vec(sinks, h, "sinks")), _ptr(gate), gate_stride, out.data_ptr(), t, b, h, g, d, dv, bs,
         int(window), int(keep_first), int(max_query_len) if max_query_len else t, float(scale), float(softcap),
-        1 if WINDOW_ATTENTION_MFMA else 0, int(chunk), 1 if crossed else 0, _dt(q), _stream()), "window_bias_attention")
+        1 if WINDOW_ATTENTION_MFMA else 0, int(chunk), cross, _dt(q), _stream()), "window_bias_attention")
     return out
 
 
