@@ -29,7 +29,7 @@ def softplus(z):
 
 
 def causal_conv(h, taps_w, bias=None):
-    """``h[T, C]``, ``taps_w[C, taps]`` (last column = the current token): zeros before the sequence's start."""
+    """``h[T, C]``, ``taps_w[C, taps]`` (newest tap last); taps that reach in front of the first token add nothing."""
     t, taps = h.shape[0], taps_w.shape[1]
     y = torch.zeros_like(h)
     for i in range(t):
@@ -62,8 +62,8 @@ def attention_mixer(h, w, p, m, eps):
     heads, groups, dim = int(m["heads"]), int(m.get("kv_heads") or m["heads"]), int(m["dim"])
     q = h @ f64(w[p + "q"]).T + f64(w[p + "q.b"])
     k = h @ f64(w[p + "k"]).T + f64(w[p + "k.b"])
-    values = k.view(t, groups, dim)                                        # the keys as projected
-    q = unit_rms(q, eps) * f64(w[p + "q.norm"])                            # over the whole projection
+    values = k.view(t, groups, dim)                                        # the un-normed key projection
+    q = unit_rms(q, eps) * f64(w[p + "q.norm"])                            # jointly over all heads
     k = unit_rms(k, eps) * f64(w[p + "k.norm"])
     if m.get("q_temp"):
         q = q * q_temperature(torch.arange(t), float(m["q_temp"]["coef"]), int(m["q_temp"]["every"])).view(-1, 1)
@@ -135,7 +135,7 @@ def mamba2_mixer(h, w, p, m, eps):
     b = xbc[:, inner:inner + groups * n].view(t, groups, n).repeat_interleave(rep, 1)
     c = xbc[:, inner + groups * n:].view(t, groups, n).repeat_interleave(rep, 1)
     y, _ = ssm_heads(x, b, c, softplus(dt + f64(w[p + "dt_bias"])), torch.exp(f64(w[p + "A_log"])), f64(w[p + "D"]))
-    y = y.reshape(t, inner) * silu(z)                                     # the gate comes before the norm
+    y = y.reshape(t, inner) * silu(z)                                     # gated first, normed second
     y = unit_rms(y.view(t, parts, inner // parts), eps).reshape(t, inner) * f64(w[p + "norm"])
     return y @ f64(w[p + "o"]).T
 

@@ -557,7 +557,7 @@ def test_values_are_the_projected_keys_and_the_temperature_steps(device, dtype):
 
 def test_mixing_head_weights_equals_mixing_crossed_outputs():
     """The definition - mix the heads' softmax weights by ``talk``, then apply head ``h``'s mixed weights to the values
-    of its own key / value head - against what the framework computes: every head's weights on every value head, then
+    of the key / value head it belongs to - against what the framework computes: every head's weights on every value head, then
     ``mix_heads``."""
     from vllm_distributed_amd.ops import torch_ref
     g = torch.Generator().manual_seed(6)
@@ -623,7 +623,7 @@ def test_convolution_tails_across_portions_first_tokens_and_stale_slots(device, 
 
 
 @pytest.mark.parametrize("device,dtype", OP_DEVICES)
-def test_the_gate_comes_before_the_grouped_norm(device, dtype):
+def test_gating_precedes_the_grouped_norm(device, dtype):
     from vllm_distributed_amd import ops
     dt = getattr(torch, dtype)
     g = torch.Generator().manual_seed(9)
@@ -640,7 +640,7 @@ def test_the_gate_comes_before_the_grouped_norm(device, dtype):
 
 @pytest.mark.parametrize("device", [pytest.param("cpu", id="cpu"), pytest.param("cuda", id="gpu", marks=pytest.mark.gpu)])
 def test_routing_rules(device):
-    """The largest ``top`` sigmoid scores are chosen; the weights are those scores times the scale, not renormalised
+    """The largest ``top`` sigmoid scores are chosen; the weights are those scores times the scale and nothing else
     (they do not sum to anything in particular)."""
     from vllm_distributed_amd.models.layers.moe import ScoredTopKMoE
     with torch.device(device):

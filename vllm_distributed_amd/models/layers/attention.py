@@ -398,9 +398,9 @@ class WindowBiasAttention(Attention):
 
 class CrossedBiasAttention(WindowBiasAttention):
     """Causal softmax attention with the logarithmic distance bias of ``WindowBiasAttention`` whose VALUES ARE ITS
-    KEYS as projected (the key rows hold the normed keys, the values the projection itself, so ``vdim = dim`` and
+    KEYS before their norm (the key rows hold the normed keys, the values the projection itself, so ``vdim = dim`` and
     there is no value projection) and whose heads exchange their softmax weights: ``weight_h <- sum_g talk[h, g]
-    weight_g``, head ``h`` then applying the mixed weights to the values of its own key / value head.  Computed as
+    weight_g``, each head then reading the values of the key / value head it belongs to with its mixed weights.  Computed as
     ``o_h = sum_g talk[h, g] * (weight_g applied to the values of h's key / value head)``: the attention kernel
     applies every query head's weights to every value head (fp32 ``[T, H, Hkv, dim]``) and ``ops.mix_heads`` sums.
     Callers norm q / k and write the cache with ``ops.joint_norm_cache``."""

@@ -85,7 +85,7 @@ class GatedDeltaRule(nn.Module):
 class SelectiveStateSpace(nn.Module):
     """A state-space recurrence in its dual (attention-like) form: per head an ``n_state x vdim`` fp32 state with
     ``S <- exp(-exp(a_log[h]) * d) * S + d * B u^T`` and ``y = S^T C + d_skip[h] * u``, where the step size
-    ``d = softplus(dt + dt_bias[h])`` comes from the token (no clamp); ``heads`` heads share ``groups`` B / C vectors
+    ``d = softplus(dt + dt_bias[h])`` comes from the token (unbounded above); ``heads`` heads share ``groups`` B / C vectors
     in runs of neighbours.  The state tensors are ``layers.short_conv.SlotState`` objects the caller owns;
     ``forward`` reads ``[u | B | C]`` from the leading columns of ``x`` and returns the fp32 heads
     ``[T, heads * vdim]`` side by side.  ``skip`` False: no ``d_skip`` term."""

@@ -625,7 +625,7 @@ class GatedMLP(nn.Module):
 class ScoredTopKMoE(FusedMoE):
     """Routed experts of the gated form ``down(silu(gate(x)) * up(x))`` behind a router whose outputs are scored one
     by one: ``score = sigmoid(router(x))``, the ``top_k`` largest scores are chosen and ARE the weights, times
-    ``route_scale``, not renormalised.  ``shared_inter > 0``: an expert of the same form that every token uses, whose
+    ``route_scale``; their sum is left as it comes.  ``shared_inter > 0``: an expert of the same form that every token uses, whose
     output ``forward`` returns beside the routed sum (the caller adds both to its residual stream in one launch).
 
     The router is fp32 (product and scores).  On the GPU in 16-bit types the experts run as two grouped GEMMs over

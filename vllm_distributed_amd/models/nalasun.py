@@ -9,7 +9,7 @@ and from model to model.  A final norm and the embedding table itself give fp32 
 
 Mixers
   * ``attention`` - ``layers.attention.CrossedBiasAttention``: grouped-query softmax attention without rotation;
-    q and k have biases and are RMS-normed over ALL their heads at once; the values are the keys as projected (no
+    q and k have biases and are RMS-normed over ALL their heads at once; the un-normed key projection doubles as the value (no
     value projection); q is scaled by ``1 + coef * ln(floor((p + 1) / every) + 1)`` at position ``p``; the score is
     ``q.k * scale - r1[h] * ln(1 + r2[h] * (i - j))``; after the softmax the heads' weights are mixed by a learned
     ``[H, H]`` matrix.

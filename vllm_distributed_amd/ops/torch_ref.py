@@ -905,7 +905,7 @@ def selective_scan(x: torch.Tensor, dt: torch.Tensor, num_heads: int, groups: in
                    slots: torch.Tensor, query_start_loc: torch.Tensor, seq_lens: torch.Tensor) -> torch.Tensor:
     """A state-space recurrence with one data-dependent decay per head over the packed rows ``x[T, C]`` =
     ``[u (H * vdim) | B (G * N) | C (G * N)]``; head ``h`` reads B / C group ``h // (H / G)``.  Per row
-    ``d = softplus(dt[t, h] + dt_bias[h])`` (no clamp), ``S <- exp(-exp(a_log[h]) * d) * S + d * B u^T`` (``S`` is
+    ``d = softplus(dt[t, h] + dt_bias[h])`` (unbounded above), ``S <- exp(-exp(a_log[h]) * d) * S + d * B u^T`` (``S`` is
     ``N x vdim``), ``y = S^T C + d_skip[h] * u``.  ``S`` is ``state[slots[i]]`` (``[slots, H, N, vdim]`` fp32) for
     sequence ``i``, taken as zero when the rows start at position 0 whatever the slot held, and left holding the state
     after the sequence's last row.  fp32 arithmetic; returns fp32 ``[T, H * vdim]``."""
