@@ -586,6 +586,8 @@ struct AttnArgs {
   int xcd_seqs;                     // > 0 (= sequences; grid.x == 1, grid.z padded to a multiple of 8): the workgroups of
                                     // one sequence are dealt to ONE of the chip's 8 dies (workgroups go to the dies in
                                     // turn by their linear number), so that what they all read is shared in its L2
+  int key_heads;                    // > 0 (crossed, decoded rows): a workgroup's wave sets take this many KEY heads, one
+                                    // each, for the same value heads, whose fragments they then share in the CU's cache
 };
 
 template <typename T, bool VEC> struct RowDot;
@@ -747,7 +749,7 @@ __global__ void window_bias_attention_kernel(AttnArgs a) {
 // value heads only): the step's weights are applied to CG value heads in turn, each with accumulators of its own, so
 // the scores and the softmax are computed once for all of them.
 template <int DT, int VT, int CG>
-__global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArgs a, const int* __restrict__ qsl,
+__global__ __launch_bounds__(CG > 1 ? 512 : 256) void window_bias_attention_mfma_kernel(AttnArgs a, const int* __restrict__ qsl,
                                                                          const int* __restrict__ seq_lens, int hp,
                                                                          int tpw, int kw) {
   using T = bf16_t;
@@ -769,12 +771,13 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   const int hchunks = (qpg + hp - 1) / hp;
   const int gy = by / hchunks, hc = by % hchunks;
   const int vchunks = a.cross ? (a.G + CG - 1) / CG : 1;
-  const int g = a.cross ? gy / vchunks : gy;                  // key head
-  const int gv0 = a.cross ? (gy % vchunks) * CG : g;          // first value head (the only one unless crossed)
-  const int tw = nwaves / kw;                     // waves over tokens
+  const int tw = nwaves / kw;                     // wave sets: over tokens, or (key_heads) over key heads
   const int wt = wave / kw, wk = wave % kw;
+  const int g = a.cross ? (a.key_heads > 0 ? (gy / vchunks) * a.key_heads + wt : gy / vchunks) : gy;       // key head
+  const int gv0 = a.cross ? (gy % vchunks) * CG : g;          // first value head (the only one unless crossed)
   const int q0 = qsl[s], n_tok = qsl[s + 1] - q0;
-  const int tok0 = (blockIdx.x * tw + wt) * tpw;  // first token (within the step's rows of the sequence) of this wave
+  // first token (within the step's rows of the sequence) of this wave
+  const int tok0 = a.key_heads > 0 ? 0 : (blockIdx.x * tw + wt) * tpw;
   if (tok0 >= n_tok && kw == 1) return;
   const bool wave_live = tok0 < n_tok;
   const int start = seq_lens[s] - n_tok;          // position of the sequence's first row in this step
@@ -936,7 +939,7 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
   // brings its sums to the common maximum, then wave 0 adds them up, one value head at a time
   if (kw > 1) {
     float* ml = lds;                                                    // [tw * kw * 64][2]
-    float* buf = lds + (long)tw * kw * 64 * 2;                          // [tw * kw * 64][4 * VT]
+    float* buf = lds + (long)tw * kw * 64 * 2;                          // [tw * (kw - 1) * 64][4 * VT]: waves wk > 0
     float* mine = ml + ((long)(wt * kw + wk) * 64 + lane) * 2;
     mine[0] = m; mine[1] = l;
     __syncthreads();
@@ -952,8 +955,8 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
     m = m_all; l = l_all;
 #pragma unroll
     for (int cc = 0; cc < CG; ++cc) {
-      float* pa = buf + ((long)(wt * kw + wk) * 64 + lane) * (4 * VT);
       if (wk > 0) {
+        float* pa = buf + ((long)(wt * (kw - 1) + wk - 1) * 64 + lane) * (4 * VT);
 #pragma unroll
         for (int c = 0; c < VT; ++c) {
           pa[4 * c] = acc[cc][c][0] * fs; pa[4 * c + 1] = acc[cc][c][1] * fs;
@@ -965,7 +968,7 @@ __global__ __launch_bounds__(256) void window_bias_attention_mfma_kernel(AttnArg
 #pragma unroll
         for (int c = 0; c < VT; ++c) acc[cc][c] *= fs;
         for (int o = 1; o < kw; ++o) {
-          const float* th = buf + ((long)(wt * kw + o) * 64 + lane) * (4 * VT);
+          const float* th = buf + ((long)(wt * (kw - 1) + o - 1) * 64 + lane) * (4 * VT);
 #pragma unroll
           for (int c = 0; c < VT; ++c) {
             acc[cc][c][0] += th[4 * c]; acc[cc][c][1] += th[4 * c + 1];
@@ -1196,6 +1199,17 @@ template <int DT, int CG> int launch_mfma(int vt, dim3 grid, dim3 block, size_t 
   return 1;
 }
 
+int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    n = v;
+  }
+  return n;
+}
+
 // value heads a workgroup of the crossed form takes: as many as share one computation of the scores without the
 // accumulators (CG * Dv / 16 vectors of four) outgrowing the register file
 int cross_group(int G, int vtiles) {
@@ -1223,7 +1237,7 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
       (bias_scale && !bias_rate) || chunk < 0 || (cross && (gate || sinks)))
     return 1;
   AttnArgs a{q, k_cache, v_cache, block_table, bt_stride, token_seq, positions, bias_scale, bias_rate, sinks, gate,
-             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap, chunk, cross ? 1 : 0, 0};
+             gate_stride, out, T, H, G, D, Dv, block_size, window, keep_first, scale, softcap, chunk, cross ? 1 : 0, 0, 0};
   const int gy = cross ? G * G : G;               // key heads, or (key head, value head) pairs
   const int qpg = H / G;
   const int dtiles = D / 32, vtiles = Dv / 16;
@@ -1235,10 +1249,18 @@ VDAMD_API int vdamd_window_bias_attention(const void* q, const void* k_cache, co
     const int hchunks = (qpg + hp - 1) / hp;
     int tw = 4, kw = 1;
     if (max_query_len <= tpw) { tw = 1; kw = 4; }          // few rows, many keys: the waves share the keys
-    const int gx = (max_query_len + tw * tpw - 1) / (tw * tpw);
-    const size_t lds = kw > 1 ? (size_t)tw * kw * 64 * (2 + 4 * vtiles) * sizeof(float) : 0;
     const int cg = cross ? (cross_group(G, vtiles) < cross ? cross_group(G, vtiles) : cross) : 1;
-    const int pairs = cross ? G * ((G + cg - 1) / cg) : G;      // (key head, group of value heads)
+    // crossed, decoded rows: the wave sets of a workgroup take 4 key heads for the same value heads and split each
+    // head's keys in two, so a value head is fetched once per workgroup instead of once per key head - where that
+    // still leaves a workgroup for every CU (fewer, longer walks over the keys lose more than the fetches save)
+    int key_heads = (cross && cg > 1 && max_query_len <= tpw && G % 4 == 0) ? 4 : 0;
+    if (key_heads > 0 && (long)B * (G / key_heads) * ((G + cg - 1) / cg) * hchunks < compute_units()) key_heads = 0;
+    if (key_heads > 0) { tw = key_heads; kw = 2; }
+    const int gx = key_heads > 0 ? 1 : (max_query_len + tw * tpw - 1) / (tw * tpw);
+    const size_t lds = kw > 1 ? (size_t)tw * 64 * (2 * kw + 4 * vtiles * (kw - 1)) * sizeof(float) : 0;
+    a.key_heads = key_heads;
+    // (key head(s), group of value heads)
+    const int pairs = cross ? (key_heads > 0 ? G / key_heads : G) * ((G + cg - 1) / cg) : G;
     dim3 grid(gx, pairs * hchunks, B), block(64 * tw * kw);
     if (cross && gx == 1 && pairs * hchunks > 1) {          // decoded rows: a sequence's workgroups on one die
       a.xcd_seqs = B;

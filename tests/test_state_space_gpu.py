@@ -141,7 +141,7 @@ def test_joint_norm_cache(dtype, h, g, d, every):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("h,g,d", [(4, 2, 32), (6, 3, 64), (4, 4, 16), (2, 1, 128), (3, 3, 24), (8, 2, 64), (8, 4, 128),
-                                   (16, 8, 32), (10, 2, 32), (5, 5, 64)])
+                                   (16, 8, 32), (10, 2, 32), (5, 5, 64), (36, 1, 32), (12, 4, 64), (12, 6, 32)])
 def test_crossed_attention_and_mixing(dtype, h, g, d):
     hip = _hip()
     gen = torch.Generator(device="cuda").manual_seed(h * 100 + d)

@@ -1309,7 +1309,7 @@ CONV_MAX_TAPS = 16
 UNIT_MAX_WIDTH = 512
 # the matrix-core attention kernel where the shape allows it (tests switch it off to run the plain kernel in bf16)
 WINDOW_ATTENTION_MFMA = os.environ.get("VDAMD_WINDOW_ATTENTION_MFMA", "1") != "0"
-CROSS_GROUP_PROMPT = int(os.environ.get("VDAMD_CROSS_GROUP_PROMPT", "2"))
+CROSS_GROUP_PROMPT = int(os.environ.get("VDAMD_CROSS_GROUP_PROMPT", "4"))
 CROSS_GROUP_DECODE = int(os.environ.get("VDAMD_CROSS_GROUP_DECODE", "2"))
 
 
@@ -1377,8 +1377,8 @@ def window_bias_attention(q, k_cache, v_cache, block_table, query_start_loc, seq
         assert gate.shape == (t, h) and gate.stride(1) == 1 and gate.dtype == q.dtype
         gate_stride = gate.stride(0)
     out_shape, out_dtype = ((t, h, g, dv), torch.float32) if crossed else ((t, h, dv), q.dtype)
-    # value heads that share one computation of the scores (measured: with four, the accumulators of four heads
-    # leave a SIMD one resident wave, and both prompt portions and decoded rows run slower than with two)
+    # value heads that share one computation of the scores: four where the rows fill the matrix cores (prompt
+    # portions); decoded rows are bound by the loads in flight, and two leave more waves resident (measured)
     cross = 0 if not crossed else (CROSS_GROUP_DECODE if max_query_len == 1 else CROSS_GROUP_PROMPT)
     assert not crossed or (gate is None and sinks is None)
     if out is None:
