@@ -168,3 +168,24 @@ def test_crossed_attention_and_mixing(dtype, h, g, d):
     plain = want[:, torch.arange(h, device="cuda"), own]
     _close(hip.mix_heads(want, torch.eye(h, device="cuda"), torch.float32), plain.reshape(want.shape[0], -1),
            torch.float32)
+
+
+@pytest.mark.parametrize("h,g,d", [(8, 4, 64), (16, 8, 32), (4, 4, 128), (12, 4, 32)])
+def test_crossed_decode_with_a_workgroup_per_cu_or_more(h, g, d):
+    """Enough decoded sequences that the launch gives a workgroup's wave sets four key heads each (bf16, key heads a
+    multiple of 4): contexts of every length from one key to several pages, sequences that are no multiple of 8."""
+    hip = _hip()
+    dtype = torch.bfloat16
+    gen = torch.Generator(device="cuda").manual_seed(h + d)
+    bs, nseq, per = 16, 300, 9
+    k, v = _caches(nseq * per, g, bs, d, dtype, gen)
+    r1 = torch.rand(h, device="cuda", generator=gen)
+    r2 = torch.rand(h, device="cuda", generator=gen)
+    table = torch.randperm(nseq * per, device="cuda", generator=gen).to(torch.int32).view(nseq, per)
+    ctx = [(7 * i) % (bs * per - 1) for i in range(nseq)]
+    qsl, sls, pos, _ = _batch([1] * nseq, ctx)
+    q = (torch.randn(nseq, h, d, device="cuda", generator=gen) * 1.5).to(dtype)
+    got = hip.window_bias_attention(q, k, v, table, qsl, sls, None, pos, 0.2, 0.0, 0, 0, r1, r2, None, None, 1, None, 0,
+                                    crossed=True)
+    want = torch_ref.crossed_bias_attention(q, k, v, table, qsl, sls, 0.2, r1, r2)
+    _close(got, want, dtype, 4)
