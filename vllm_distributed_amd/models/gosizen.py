@@ -41,7 +41,7 @@ from ..parallel.state import get_pp_group, get_tensor_model_parallel_world_size
 from .layers.attention import (Attention, ResidualRMSNorm, RowLatentAttention, WindowBiasAttention, get_forward_context,
                                rotary_frequencies)
 from .layers.linear import ColumnParallelLinear, ReplicatedLinear, RowParallelLinear, VocabParallelEmbedding
-from .layers.linear_attention import GatedDeltaRule
+from .layers.linear_attention import DeltaRuleMixer
 from .layers.moe import BiasedTopKMoE
 from .layers.short_conv import ShortConv, SlotState
 from .utils import IntermediateTensors, materialize
@@ -167,43 +167,6 @@ class ChunkedConvAttention(nn.Module):
             ctx.positions, self.heads, self.kv_heads, self.dim, self.vdim, None, None, self.eps, None, None, False,
             attn.k_cache, attn.v_cache, md.slot_mapping, md.num_prefills > 0, self.inv_freq)
         ops.sigmoid_mul(attn.forward_cached(q), x[:, self.channels:], self.out_scale, out=out)
-
-
-class DeltaRuleMixer(nn.Module):
-    """The right half of a parallel mixer; writes ``scale * normed, gated heads`` into the columns it is given."""
-
-    def __init__(self, width: int, m: dict, eps: float, layer_idx: int, dtype: torch.dtype, passes: int, scale: float):
-        super().__init__()
-        self.heads, self.qk_heads = int(m["heads"]), int(m.get("kv_heads") or m["heads"])
-        self.dim, self.vdim = int(m["dim"]), int(m.get("vdim") or m["dim"])
-        self.decay_rank, self.gate_rank = int(m["decay_rank"]), int(m["gate_rank"])
-        self.eps, self.dtype, self.out_scale = eps, dtype, float(scale)
-        qs, vs = self.qk_heads * self.dim, self.heads * self.vdim
-        self.channels, self.out_cols = 2 * qs + vs, vs
-        self.proj = ColumnParallelLinear(width, [qs, qs, vs, self.heads, self.decay_rank, self.gate_rank], False, dtype)
-        self.a2 = ReplicatedLinear(self.decay_rank, self.heads * self.dim, False, dtype)
-        self.g2 = ReplicatedLinear(self.gate_rank, vs, False, dtype)
-        self.conv = ShortConv([qs, qs, vs], int(m.get("conv") or 1), dtype)
-        self.rule = GatedDeltaRule(self.heads, self.qk_heads, self.dim, self.vdim, layer_idx)
-        self.conv_states = [SlotState((max(self.conv.taps - 1, 1), self.channels)) for _ in range(passes)]
-        self.rule_states = [SlotState(self.rule.per_slot_shape(), torch.float32) for _ in range(passes)]
-        self.norm = _f32(self.vdim)
-
-    def forward(self, h: torch.Tensor, index: int, out: torch.Tensor) -> None:
-        ctx = get_forward_context()
-        md = ctx.attn_metadata
-        x = self.proj(h)
-        c = self.channels
-        dt = self.a2(x[:, c + self.heads:c + self.heads + self.decay_rank])
-        gate = self.g2(x[:, c + self.heads + self.decay_rank:])
-        if md is None:                    # memory-profiling pass: no state
-            out.zero_()
-            return
-        rows = None if md.num_prefills == 0 else md.token_rows(ctx.positions)[0]
-        qkv = ops.short_conv_act(x, c, self.conv.weight_t, self.conv_states[index].state, md.state_slots,
-                                 md.query_start_loc, md.seq_lens, rows, ctx.positions, True, md.num_prefills > 0)
-        o = self.rule(qkv, x[:, c:c + self.heads], dt, self.rule_states[index].state)
-        ops.gated_rms_norm(o, self.norm, gate, self.eps, self.dtype, group=self.vdim, scale=self.out_scale, out=out)
 
 
 class ParallelMixer(nn.Module):

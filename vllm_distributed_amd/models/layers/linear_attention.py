@@ -16,6 +16,8 @@ import torch.nn as nn
 
 from ... import ops
 from .attention import get_forward_context
+from .linear import ColumnParallelLinear, ReplicatedLinear
+from .short_conv import ShortConv, SlotState
 
 
 class DecayLinearAttention(nn.Module):
@@ -116,3 +118,45 @@ class SelectiveStateSpace(nn.Module):
         return ops.selective_scan(x, dt, self.heads, self.groups, self.vdim, self.n_state, self.a_log, self.dt_bias,
                                   self.d_skip, state, md.state_slots, md.query_start_loc, md.seq_lens,
                                   md.max_query_len)
+
+
+class DeltaRuleMixer(nn.Module):
+    """Everything of a gated-delta-rule mixer between its normed input and its output projection: one fused projection
+    ``[q | k | v | beta | decay rank | gate rank]``, the two low-rank up-projections, convolution + SiLU over
+    ``[q | k | v]``, the recurrence, and the per-head RMS norm times the sigmoid gate.  ``passes``: how many times the
+    layer runs in a forward pass over these weights (each run with convolution tails and a state of its own);
+    ``forward`` writes ``scale * normed, gated heads`` into the columns it is given, so a caller may fuse several
+    mixers' output projections."""
+
+    def __init__(self, width: int, m: dict, eps: float, layer_idx: int, dtype: torch.dtype, passes: int, scale: float):
+        super().__init__()
+        self.heads, self.qk_heads = int(m["heads"]), int(m.get("kv_heads") or m["heads"])
+        self.dim, self.vdim = int(m["dim"]), int(m.get("vdim") or m["dim"])
+        self.decay_rank, self.gate_rank = int(m["decay_rank"]), int(m["gate_rank"])
+        self.eps, self.dtype, self.out_scale = eps, dtype, float(scale)
+        qs, vs = self.qk_heads * self.dim, self.heads * self.vdim
+        self.channels, self.out_cols = 2 * qs + vs, vs
+        self.proj = ColumnParallelLinear(width, [qs, qs, vs, self.heads, self.decay_rank, self.gate_rank], False, dtype)
+        self.a2 = ReplicatedLinear(self.decay_rank, self.heads * self.dim, False, dtype)
+        self.g2 = ReplicatedLinear(self.gate_rank, vs, False, dtype)
+        self.conv = ShortConv([qs, qs, vs], int(m.get("conv") or 1), dtype)
+        self.rule = GatedDeltaRule(self.heads, self.qk_heads, self.dim, self.vdim, layer_idx)
+        self.conv_states = [SlotState((max(self.conv.taps - 1, 1), self.channels)) for _ in range(passes)]
+        self.rule_states = [SlotState(self.rule.per_slot_shape(), torch.float32) for _ in range(passes)]
+        self.norm = nn.Parameter(torch.zeros(self.vdim, dtype=torch.float32), requires_grad=False)
+
+    def forward(self, h: torch.Tensor, index: int, out: torch.Tensor) -> None:
+        ctx = get_forward_context()
+        md = ctx.attn_metadata
+        x = self.proj(h)
+        c = self.channels
+        dt = self.a2(x[:, c + self.heads:c + self.heads + self.decay_rank])
+        gate = self.g2(x[:, c + self.heads + self.decay_rank:])
+        if md is None:                    # memory-profiling pass: no state
+            out.zero_()
+            return
+        rows = None if md.num_prefills == 0 else md.token_rows(ctx.positions)[0]
+        qkv = ops.short_conv_act(x, c, self.conv.weight_t, self.conv_states[index].state, md.state_slots,
+                                 md.query_start_loc, md.seq_lens, rows, ctx.positions, True, md.num_prefills > 0)
+        o = self.rule(qkv, x[:, c:c + self.heads], dt, self.rule_states[index].state)
+        ops.gated_rms_norm(o, self.norm, gate, self.eps, self.dtype, group=self.vdim, scale=self.out_scale, out=out)

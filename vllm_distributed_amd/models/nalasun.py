@@ -36,10 +36,9 @@ import torch.nn as nn
 from .. import ops
 from ..config import VllmConfig
 from ..parallel.state import get_pp_group, get_tensor_model_parallel_world_size
-from .gosizen import DeltaRuleMixer
 from .layers.attention import Attention, CrossedBiasAttention, ResidualRMSNorm, get_forward_context
 from .layers.linear import ColumnParallelLinear, RowParallelLinear, VocabParallelEmbedding
-from .layers.linear_attention import SelectiveStateSpace
+from .layers.linear_attention import DeltaRuleMixer, SelectiveStateSpace
 from .layers.moe import ScoredTopKMoE
 from .layers.short_conv import ShortConv, SlotState
 from .utils import IntermediateTensors, materialize
