@@ -775,6 +775,25 @@ def test_dummy_weights_and_config_keys():
         assert len(out[0].outputs[0].token_ids) == 4
 
 
+def test_sizes_that_only_tensor_shapes_state(tmp_path_factory, tmp_path):
+    """A config that leaves out what the tensors' shapes say anyway - the taps of every convolution, the low-rank
+    widths, the number of positions - loads and computes the same model."""
+    from safetensors.torch import save_file
+    path, cfg, w = model_dir("paged", tmp_path_factory)
+    bare = json.loads(json.dumps(cfg))
+    bare.pop("canon")
+    bare.pop("max_positions")
+    for spec in bare["layers"]:
+        spec["mixer"].pop("conv", None)
+    d = tmp_path / "bare"
+    d.mkdir()
+    save_file({k: v.contiguous() for k, v in w.items()}, str(d / "model.safetensors"))
+    (d / "config.json").write_text(json.dumps(bare))
+    toks = tokens_for(cfg, 40, 70)
+    got = run_schedule(str(d), portions(toks, [17, 1], "r"), "float32", "cpu", max_tokens=64, tmp=tmp_path)
+    check(got, "paged", cfg, w, {"r": toks}, 2e-4)
+
+
 def test_the_trace_runner_as_a_program(tmp_path_factory, tmp_path):
     import subprocess
     import sys

@@ -48,6 +48,13 @@ def _f32(*shape: int) -> nn.Parameter:
     return nn.Parameter(torch.zeros(shape, dtype=torch.float32), requires_grad=False)
 
 
+def _taps(shapes: Dict[str, Tuple[int, ...]], tensor: str, stated) -> int:
+    """Taps of a convolution: the checkpoint tensor's second dimension where there is one, else what the config
+    states."""
+    shape = shapes.get(tensor)
+    return int(shape[1]) if shape is not None and len(shape) == 2 else int(stated or 0)
+
+
 def _conv_rows(md, positions):
     """The sequence of every row of the step (None in a pure decode batch: row ``t`` is sequence ``t``)."""
     return None if md.num_prefills == 0 else md.token_rows(positions)[0]
@@ -102,6 +109,7 @@ class ChannelDeltaMixer(nn.Module):
                     raise ValueError(f"layer {layer_idx}: neither the config ({key}) nor a checkpoint tensor "
                                      f"(mix.{tensor}) gives the width of the low-rank projection")
                 m[key] = int(shape[0])
+        m["conv"] = _taps(shapes, f"l{layer_idx}.mix.q.conv", m.get("conv")) or 1
         self.dtype = dtype
         self.inner = DeltaRuleMixer(width, m, eps, layer_idx, dtype, 1, 1.0)
         self.o = RowParallelLinear(self.inner.out_cols, width, False, dtype)
@@ -116,7 +124,8 @@ class ChannelDeltaMixer(nn.Module):
 
 
 class StateSpaceMixer(nn.Module):
-    def __init__(self, width: int, m: dict, eps: float, layer_idx: int, dtype: torch.dtype):
+    def __init__(self, width: int, m: dict, eps: float, layer_idx: int, dtype: torch.dtype,
+                 shapes: Dict[str, Tuple[int, ...]]):
         super().__init__()
         heads, vdim, n, groups = int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m.get("groups") or 1)
         self.inner_cols, self.eps, self.dtype = heads * vdim, eps, dtype
@@ -128,7 +137,8 @@ class StateSpaceMixer(nn.Module):
         bc = groups * n
         # [z | x | B | C | dt]
         self.proj = ColumnParallelLinear(width, [self.inner_cols, self.inner_cols, bc, bc, heads], False, dtype)
-        self.conv = ShortConv([self.inner_cols, bc, bc], int(m.get("conv") or 1), dtype, bias=True)
+        self.conv = ShortConv([self.inner_cols, bc, bc], _taps(shapes, f"l{layer_idx}.mix.conv", m.get("conv")) or 1,
+                              dtype, bias=True)
         self.conv_state = SlotState((max(self.conv.taps - 1, 1), self.conv.channels))
         self.ssm_state = SlotState(self.ssm.per_slot_shape(), torch.float32)
         self.norm = _f32(self.inner_cols)
@@ -160,7 +170,7 @@ def _make_mixer(width: int, spec: dict, eps: float, layer_idx: int, dtype: torch
     if kind == "channel_delta":
         return ChannelDeltaMixer(width, m, eps, layer_idx, dtype, shapes)
     if kind == "mamba2":
-        return StateSpaceMixer(width, m, eps, layer_idx, dtype)
+        return StateSpaceMixer(width, m, eps, layer_idx, dtype, shapes)
     raise ValueError(f"layer {layer_idx}: unknown mixer type {kind!r}")
 
 
@@ -222,18 +232,21 @@ class NalasunForCausalLM(nn.Module):
                                       "state is not sharded")
         self.is_first = self.is_last = True
         width, eps = int(cfg["width"]), float((cfg.get("norm") or {}).get("eps", 1e-5))
-        taps = int((cfg.get("canon") or {}).get("taps") or 0)
         specs = cfg["layers"]
         if not specs:
             raise ValueError("a Nalasun model needs at least one layer")
         self.width, self.eps, self.vocab = width, eps, int(cfg["vocab"])
         self.start_layer, self.end_layer = 0, len(specs)
         self.embed = VocabParallelEmbedding(self.vocab, width, dtype)
-        self.pos = nn.Embedding(int(cfg["max_positions"]), width, dtype=dtype)
-        self.pos.weight.requires_grad_(False)
         from ..config import resolve_model_path
         from .loader import checkpoint_tensor_shapes
         shapes = {} if mc.load_format == "dummy" else checkpoint_tensor_shapes(resolve_model_path(mc.model))
+        taps = _taps(shapes, "l0.canon1", (cfg.get("canon") or {}).get("taps"))
+        positions = int(cfg.get("max_positions") or (shapes.get("pos") or (0,))[0])
+        if positions <= 0:
+            raise ValueError("neither the config (max_positions) nor a checkpoint tensor (pos) gives the number of positions")
+        self.pos = nn.Embedding(positions, width, dtype=dtype)
+        self.pos.weight.requires_grad_(False)
         self.layers = nn.ModuleList(NalasunLayer(width, s, eps, taps, i, dtype, shapes) for i, s in enumerate(specs))
         self.final_norm = ResidualRMSNorm(width, eps, dtype)
         self.trace_residual: Optional[List[torch.Tensor]] = None      # tests: the residual stream after every layer
